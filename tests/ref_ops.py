@@ -144,12 +144,16 @@ def _gelu_tanh(g):
     return 0.5 * g * (1.0 + torch.tanh(0.7978845608 * (g + 0.044715 * g * g * g)))
 
 
-def gated_linear(x, w_packed, inter, activation, out_dtype):
-    act = {"gelu_tanh": _gelu_tanh, "silu": lambda g: g * torch.sigmoid(g), "relu": torch.relu}[activation]
+def gated_linear(x, w_packed, inter, activation, out_dtype, limit=None, up_shift=0.0):
+    """limit: the gate sum is cut at it from above and the up sum from both sides, before the activation."""
+    act = {"gelu_tanh": _gelu_tanh, "silu": lambda g: g * torch.sigmoid(g), "relu": torch.relu,
+           "quick_gelu": lambda g: g * torch.sigmoid(1.702 * g)}[activation]
     y = x.float() @ w_packed.float().T                     # [M, 2 * ip]
     y = y.reshape(x.shape[0], -1, 2, GROUP)
     g, u = y[:, :, 0, :].reshape(x.shape[0], -1), y[:, :, 1, :].reshape(x.shape[0], -1)
-    return (act(g) * u)[:, :inter].to(out_dtype).contiguous()
+    if limit is not None:
+        g, u = torch.clamp(g, max=limit), torch.clamp(u, -limit, limit)
+    return (act(g) * (u + up_shift))[:, :inter].to(out_dtype).contiguous()
 
 
 def _rotate(x, pos, inv_freq, rotary_dim, pairing="halves"):
@@ -197,17 +201,24 @@ def kv_write(k, v, KV, hd, row_seq, row_pos, new_len, table, k_pool, v_pool, row
     _cache_rows(k, v, row_seq, row_pos, new_len, table, k_pool, v_pool, rows_cap)
 
 
-def _attend(qrow, keys, vals, scale, softcap):
-    """qrow [hd], keys/vals [n, hd], fp32."""
+def _attend(qrow, keys, vals, scale, softcap, sink=None):
+    """qrow [hd], keys/vals [n, hd], fp32.  sink: a score without key or value that joins the denominator."""
     s = (keys @ qrow) * scale
     if softcap:
         s = softcap * torch.tanh(s / softcap)
+    if sink is not None:
+        return torch.softmax(torch.cat([s, sink.reshape(1).float()]), dim=0)[:-1] @ vals
     p = torch.softmax(s, dim=0)
     return p @ vals
 
 
+def _first_seen(p, window, chunk):
+    lo = 0 if not window else max(0, p - window + 1)
+    return max(lo, (p // chunk) * chunk) if chunk else lo
+
+
 def attention_prefill(q, k, v, H, KV, hd, cu_rows, max_count, scale, softcap, window, out_dtype, row_seq=None, row_pos=None,
-                      cached=None, shape=0, wide_weights=False):
+                      cached=None, shape=0, wide_weights=False, chunk=0, head_scale=None, sink=None):
     """k, v: the step's own rows.  cached None: every sequence starts at position 0.  Else cached = (new_len, table,
     k_pool, v_pool, rows_cap): sequence i's first row stands at new_len[i] - its count, and the positions before it are
     read from the cache as it is."""
@@ -222,7 +233,7 @@ def attention_prefill(q, k, v, H, KV, hd, cu_rows, max_count, scale, softcap, wi
             new_len, table, k_pool, v_pool, rows_cap = cached
             page = k_pool.shape[2]
             start = int(new_len[i]) - (b - a)
-            first = max(0, start - (window - 1)) if window else 0       # the earliest position any query of the step sees
+            first = _first_seen(start, window, chunk)                    # the earliest position any query of the step sees
             pos = torch.arange(first, start)
             rows = pos % rows_cap if rows_cap else pos
             pages = table[i].long()[rows // page]
@@ -231,9 +242,11 @@ def attention_prefill(q, k, v, H, KV, hd, cu_rows, max_count, scale, softcap, wi
             vals = torch.cat([torch.zeros(first, KV, hd), v_pool[pages, :, rows % page, :].float().cpu(), vf[a:b].cpu()]).to(q.device)
         for r in range(a, b):
             p = start + r - a
-            lo = 0 if not window else max(0, p - window + 1)
+            lo = _first_seen(p, window, chunk)
             for h in range(H):
-                out[r, h * hd:(h + 1) * hd] = _attend(qf[r, h], keys[lo:p + 1, h // g], vals[lo:p + 1, h // g], scale, softcap)
+                out[r, h * hd:(h + 1) * hd] = _attend(qf[r, h], keys[lo:p + 1, h // g], vals[lo:p + 1, h // g],
+                                                      scale * (float(head_scale[h]) if head_scale is not None else 1.0), softcap,
+                                                      None if sink is None else sink[h])
     return out.to(out_dtype)
 
 
@@ -241,7 +254,8 @@ def decode_splits(n, KV, hd, keys):
     return 1
 
 
-def attention_decode(q, H, KV, hd, new_len, table, k_pool, v_pool, rows_cap, scale, softcap, window, out_dtype, max_keys=None, splits=None, head_groups=None):
+def attention_decode(q, H, KV, hd, new_len, table, k_pool, v_pool, rows_cap, scale, softcap, window, out_dtype, max_keys=None, splits=None, head_groups=None,
+                     chunk=0, head_scale=None, sink=None):
     n = q.shape[0]
     page = k_pool.shape[2]
     out = torch.zeros((n, H * hd), dtype=torch.float32, device=q.device)
@@ -249,7 +263,7 @@ def attention_decode(q, H, KV, hd, new_len, table, k_pool, v_pool, rows_cap, sca
     g = H // KV
     for i in range(n):
         p = int(new_len[i]) - 1
-        lo = 0 if not window else max(0, p - window + 1)
+        lo = _first_seen(p, window, chunk)
         pos = torch.arange(lo, p + 1)
         rows = pos % rows_cap if rows_cap else pos
         pages = table[i].long()[rows // page]
@@ -257,7 +271,9 @@ def attention_decode(q, H, KV, hd, new_len, table, k_pool, v_pool, rows_cap, sca
         keys = k_pool[pages, :, rows % page, :].float()          # [n_keys, KV, hd]
         vals = v_pool[pages, :, rows % page, :].float()
         for h in range(H):
-            out[i, h * hd:(h + 1) * hd] = _attend(qf[i, h], keys[:, h // g], vals[:, h // g], scale, softcap)
+            out[i, h * hd:(h + 1) * hd] = _attend(qf[i, h], keys[:, h // g], vals[:, h // g],
+                                                  scale * (float(head_scale[h]) if head_scale is not None else 1.0), softcap,
+                                                  None if sink is None else sink[h])
     return out.to(out_dtype)
 
 
@@ -339,6 +355,79 @@ def ssd_scan(xbc, z, dt, dt_bias, a_log, skip, state, slot_ids, cu_rows, max_cou
         state[slot] = S
     zf = z.float()
     return y.reshape(m, inner) * (zf * torch.sigmoid(zf))
+
+
+def shift_mix(x, mu, state, slot_ids, cu_rows, row_seq, one_row_each=False):
+    """out[s, r] = x[r] + (x[r - 1] - x[r]) * mu[s] within each sequence; the row before a sequence's first row of the
+    step is state[slot] (float32 [slots, D]), which then takes the sequence's last row."""
+    xf = x.float()
+    before = torch.empty_like(xf)
+    for i in range(len(cu_rows) - 1):
+        a, b, slot = int(cu_rows[i]), int(cu_rows[i + 1]), int(slot_ids[i])
+        before[a] = state[slot]
+        before[a + 1:b] = xf[a:b - 1]
+        state[slot] = xf[b - 1]
+    return (xf[None] + (before - xf)[None] * mu[:, None, :]).to(x.dtype)
+
+
+def unary_(x, name):
+    """In place: x <- tanh(x)."""
+    assert name == "tanh"
+    x.copy_(torch.tanh(x.float()).to(x.dtype))
+    return x
+
+
+def time_mix_scan(r, k, v, log_rate, w0, bonus, state, slot_ids, cu_rows, max_count, heads, dim):
+    """o = (S + diag(bonus) k v^T)^T r, then S <- diag(w) S + k v^T with w = exp(-exp(log_rate + w0)), row after row of
+    every sequence from state[slot] [heads, dim, dim], which is left updated.  float32 [M, heads dim]."""
+    m = r.shape[0]
+    rf, kf, vf = (t.float().reshape(m, heads, dim) for t in (r, k, v))
+    w = torch.exp(-torch.exp(log_rate.float() + w0)).reshape(m, heads, dim)
+    y = torch.empty((m, heads, dim), dtype=torch.float32, device=r.device)
+    for i in range(len(cu_rows) - 1):
+        slot = int(slot_ids[i])
+        S = state[slot].clone()
+        for t in range(int(cu_rows[i]), int(cu_rows[i + 1])):
+            kv = kf[t][:, :, None] * vf[t][:, None, :]
+            y[t] = torch.einsum("hkv,hk->hv", S + bonus[:, :, None] * kv, rf[t])
+            S = w[t][:, :, None] * S + kv
+        state[slot] = S
+    return y.reshape(m, heads * dim)
+
+
+def matrix_memory_scan(q, k, v, gates, cap, q_scale, memory, normalizer, maximum, slot_ids, cu_rows, max_count, heads, dk, dv):
+    """gates float32 [M, 2 heads]: the input and forget gates' sums.  i = cap tanh(. / cap), f = logsigmoid(cap tanh(. / cap)),
+    m' = max(f + m, i), S <- e^(f + m - m') S + e^(i - m') k v^T, n likewise with k, o = S^T q' / (max(|n . q'|, e^(-m')) + 1e-6)
+    with q' = q q_scale; the states [slots, heads, dk, dv], [slots, heads, dk], [slots, heads] are left updated."""
+    M = q.shape[0]
+    qf, kf, vf = q.float().reshape(M, heads, dk) * q_scale, k.float().reshape(M, heads, dk), v.float().reshape(M, heads, dv)
+    gi = cap * torch.tanh(gates[:, :heads].float() / cap)
+    gf = torch.nn.functional.logsigmoid(cap * torch.tanh(gates[:, heads:].float() / cap))
+    y = torch.empty((M, heads, dv), dtype=torch.float32, device=q.device)
+    for s in range(len(cu_rows) - 1):
+        slot = int(slot_ids[s])
+        S, n, mx = memory[slot].clone(), normalizer[slot].clone(), maximum[slot].clone()
+        for t in range(int(cu_rows[s]), int(cu_rows[s + 1])):
+            new = torch.maximum(gf[t] + mx, gi[t])
+            keep, take = torch.exp(gf[t] + mx - new), torch.exp(gi[t] - new)
+            S = keep[:, None, None] * S + take[:, None, None] * kf[t][:, :, None] * vf[t][:, None, :]
+            n = keep[:, None] * n + take[:, None] * kf[t]
+            mx = new
+            den = torch.maximum((n * qf[t]).sum(-1).abs(), torch.exp(-mx)) + 1e-6
+            y[t] = torch.einsum("hkv,hk->hv", S, qf[t]) / den[:, None]
+        memory[slot], normalizer[slot], maximum[slot] = S, n, mx
+    return y.reshape(M, heads * dv)
+
+
+def head_norm_gate(y, gain, g, eps, heads, activation, out_dtype):
+    """Every head's part of a row over its root mean square, times the gain, times act(g): sigmoid(g) or silu(g)."""
+    gf = g.float()
+    act = torch.sigmoid(gf) if activation == "sigmoid" else gf * torch.sigmoid(gf)
+    return (_norm(y, gain, eps, heads) * act).to(out_dtype)
+
+
+def weighted_sum(a, wa, b, wb):
+    return wa * a.float() + wb * b.float()
 
 
 def pair_norm_mean(a, b, gain_a, gain_b, eps):

@@ -2,3 +2,4 @@ from .base import ConfigError, ModelConfig, key, read_config_json, architecture_
 from .gemma2 import Gemma2Config   # noqa: F401
 from .golepel import GolepelConfig   # noqa: F401
 from .lutovik import LutovikConfig   # noqa: F401
+from .besulix import BesulixConfig   # noqa: F401

@@ -17,6 +17,8 @@ class TensorSpec:
     shape: tuple
     init: str = "matrix"            # "matrix", "norm", "embedding": which sigma; "gain": one plus "norm"; "zeros"; "ones"
     dtype: str = "float"            # "float": kept as stored (bf16, or fp32 if stored so); "int": int32 table
+    free: tuple = ()                # dimensions whose size the checkpoint gives (no configuration key names it): `shape` there
+                                    # holds what a random model takes, and the part reads the real size when it binds
 
 
 @dataclasses.dataclass

@@ -20,6 +20,15 @@ the same.  A step that continues sequences by several tokens, or mixes starting 
 over the cached positions its queries still see, read in place through the page table, plus its own rows (the
 reference's multi-token step walks its cache from any position: runtime/src/lib.rs:676-720,
 runtime/cuda/codebook_gemv.cu:410-440), and caches its own rows after the attention.
+
+Further parameters, none of which the reference has: biases on the q, k and v projections; `chunk` C, with which the
+query at position p sees only the keys t <= p of its own chunk, floor(t / C) = floor(p / C), chunks counted from the
+sequence's first position (the cache then keeps a ring of C positions); a temperature per head that multiplies its
+scores; a sink per head, a learned score without key or value whose exponential joins the softmax's denominator once;
+and `value_rotation` theta: the value of position t is turned by t over all its elements like a key (pairs (d, d +
+value_dim / 2), frequencies theta^(-2d / value_dim)) before it is cached, and a head's output at position p is turned
+back by -p, so that the weighted sum is read in the query's frame.  With any of the last four the step runs on the
+plain kernel, which keeps scores and weights in float32.
 """
 from ..cache.store import TokenSpec
 from ..models.spec import TensorSpec
@@ -31,12 +40,16 @@ class Attention(Mixer):
     def __init__(self, hidden_size, num_heads, num_kv_heads, head_dim, query_scale,
                  softcap=None, window=None, position=("none", {}), value_dim=None, output_gate=False, own_kv=True,
                  precise_weights=False,
-                 tensors=("q_proj.weight", "k_proj.weight", "v_proj.weight", "o_proj.weight", "g_proj.weight")):
+                 tensors=("q_proj.weight", "k_proj.weight", "v_proj.weight", "o_proj.weight", "g_proj.weight"),
+                 bias_suffix=None, chunk=None, head_temperature=None, sink=None, value_rotation=None):
         """value_dim: elements of a value head when they differ from a key's head_dim.  output_gate: the heads' outputs
         are multiplied by sigmoid(W_g x) before the output projection.  own_kv False: the layer has no key and value
         projections; its schedule entry names the run whose cache it reads.  precise_weights: the softmax weights meet
         the values with 16 bits of mantissa or more in every kernel (the kernel of many queries rounds them to bfloat16
-        otherwise; a decode step's are float32 anyway).  tensors: local names of W_q, W_k, W_v, W_o (and W_g)."""
+        otherwise; a decode step's are float32 anyway).  tensors: local names of W_q, W_k, W_v, W_o (and W_g).
+        bias_suffix: q, k and v have biases, named like their matrices with this suffix.  chunk: positions per chunk.
+        head_temperature, sink: local names of float vectors [heads].  value_rotation: the base theta of the values'
+        rotation by their position."""
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads are no multiple of {num_kv_heads} kv heads")
         self.hidden_size = hidden_size
@@ -58,6 +71,22 @@ class Attention(Mixer):
         self.position = build_part("position", position)
         if self.position.rotary_dim > head_dim:
             raise ValueError(f"rotary_dim {self.position.rotary_dim} exceeds head_dim {head_dim}")
+        self.bias_suffix = bias_suffix
+        self.chunk = int(chunk) if chunk else 0
+        self.temperature_name, self.sink_name = head_temperature, sink
+        self.value_position = None
+        if value_rotation is not None:
+            self.value_position = build_part("position", ("rope", {"rotary_dim": self.value_dim, "theta": value_rotation}))
+        self.output_dtype = None         # a mixer that holds this one may ask for its last product in another dtype
+        # the kernels of the matrix cores know none of these: such an attention runs on the plain kernel
+        self.plain_only = bool(self.chunk or head_temperature or sink or value_rotation is not None)
+        if self.plain_only and (self.output_gate or not self.own_kv):
+            raise ValueError("chunks, temperatures, sinks and rotated values go with an ungated attention on its own cache")
+
+    @property
+    def reach(self):
+        """Positions back (the query's own included) that a query can see: the window, the chunk, or 0 for all."""
+        return min((n for n in (self.window, self.chunk) if n), default=0)
 
     def tensor_specs(self):
         n, d = self.names, self.hidden_size
@@ -68,11 +97,18 @@ class Attention(Mixer):
             specs[n["v"]] = TensorSpec((self.num_kv_heads * self.value_dim, d))
         if self.output_gate:
             specs[n["g"]] = TensorSpec((self.num_heads * self.value_dim, d))
+        if self.bias_suffix:
+            for s in ("q", "k", "v") if self.own_kv else ("q",):
+                specs[n[s] + self.bias_suffix] = TensorSpec((specs[n[s]].shape[0],), init="norm")
+        if self.temperature_name:
+            specs[self.temperature_name] = TensorSpec((self.num_heads,), init="gain")
+        if self.sink_name:
+            specs[self.sink_name] = TensorSpec((self.num_heads,), init="norm")
         return specs
 
     def cache_spec(self):
         per_token = (self.num_kv_heads, self.row)
-        return TokenSpec.of(self.window or None, k=per_token, v=per_token)
+        return TokenSpec.of(self.reach or None, k=per_token, v=per_token)
 
     def _heads(self, w, heads, size, turned=False):
         """[heads * size, d] -> [heads * row, d]: zero rows fill a head up to `row`.  turned: a rotation of neighbouring
@@ -104,11 +140,29 @@ class Attention(Mixer):
             w_o = w_o.reshape(-1, H * self.row).contiguous()
         self.w_o = rt.matrix(w_o)
         self.inv_freq = self.position.inv_freq(rt.device)
+        self.b_qkv = None
+        if self.bias_suffix:
+            sides = [("q", H, self.head_dim, True)] + ([("k", KV, self.head_dim, True), ("v", KV, self.value_dim, False)] if self.own_kv else [])
+            self.b_qkv = torch.cat([self._heads(tensors[n[s] + self.bias_suffix].reshape(-1, 1), heads, size, turned=t).reshape(-1)
+                                    for s, heads, size, t in sides]).float().contiguous()
+        self.temperature = tensors[self.temperature_name].float().contiguous() if self.temperature_name else None
+        self.sink = tensors[self.sink_name].float().contiguous() if self.sink_name else None
+        self.value_freq = self.value_back = None
+        if self.value_position is not None:
+            self.value_freq = self.value_position.inv_freq(rt.device)
+            self.value_back = (-self.value_freq).contiguous()            # the same angles the other way round
 
     def _project_out(self, ctx, x, out):
         if self.output_gate:
             ctx.ops.mul_sigmoid(out, ctx.ops.linear(x, self.w_g, ctx.dtype))
+        if self.output_dtype is not None:
+            return ctx.ops.linear(out, self.w_o, self.output_dtype)
         return ctx.ops.linear(out, self.w_o, ctx.dtype, defer=True)
+
+    def _turn(self, ctx, rows, heads, freq):
+        """Turn every head of `rows` by its position, over the values' elements, in place."""
+        ctx.ops.rope_kv_write(rows, None, None, heads, 0, self.row, freq, self.value_dim, ctx.row_seq, ctx.row_pos, ctx.new_len,
+                              None, None, None, 0, write=False)
 
     def forward(self, ctx, x, site):
         ops = ctx.ops
@@ -118,31 +172,38 @@ class Attention(Mixer):
         if owns_cache and not self.own_kv:
             raise ValueError("an attention without key and value projections must read another run's cache")
         w_in = self.w_qkv if owns_cache else self.w_qkv[:Q]          # a run on another run's cache projects its queries only
-        if site.spec.window is not None and not 0 < self.window <= site.spec.window:
-            raise ValueError(f"this attention sees {self.window or 'all'} keys back, the cache it reads keeps {site.spec.window}")
+        if site.spec.window is not None and not 0 < self.reach <= site.spec.window:
+            raise ValueError(f"this attention sees {self.reach or 'all'} keys back, the cache it reads keeps {site.spec.window}")
         if site.spec.shape_of("k") != (KV, hd):
             raise ValueError(f"the cache read here keeps keys of {site.spec.shape_of('k')}, this layer needs {(KV, hd)}")
         table = ctx.page_table(site.group_index)
         k_pool, v_pool = site.tensor("k"), site.tensor("v")         # [pages, kv_heads, page, row]
         rows_cap = site.rows_cap or 0
-        if ctx.mode == "decode" and ops.fuses_decode_step(ctx.dtype, H, KV, hd, k_pool):
+        bias = None if self.b_qkv is None else (self.b_qkv if owns_cache else self.b_qkv[:Q])
+        # what the plain kernel takes beyond the others: see the module's text
+        more = dict(chunk=self.chunk, head_scale=self.temperature, sink=self.sink) if self.plain_only else {}
+        if ctx.mode == "decode" and bias is None and not self.plain_only and ops.fuses_decode_step(ctx.dtype, H, KV, hd, k_pool):
             # one launch rotates, writes the cache and attends; the projections may stay in K slices until then
             qkv = ops.linear(x, w_in, ctx.dtype, defer=True)
             out = ops.attention_decode_step(qkv, H, KV, hd, self.inv_freq, self.position.rotary_dim, ctx.new_len,
                                             table, k_pool, v_pool, rows_cap, self.query_scale, self.softcap,
                                             self.window, ctx.dtype, max_keys=ctx.max_rows_visible(site), write_kv=owns_cache)
             return self._project_out(ctx, x, out)
-        qkv = ops.linear(x, w_in, ctx.dtype)
+        qkv = ops.linear(x, w_in, ctx.dtype, bias=bias) if bias is not None else ops.linear(x, w_in, ctx.dtype)
         if owns_cache:
             q, k, v = qkv[:, :Q], qkv[:, Q:Q + KVD], qkv[:, Q + KVD:]
         else:
             q, k, v = qkv, None, None
+        if self.value_freq is not None:
+            self._turn(ctx, v, KV, self.value_freq)
         if ctx.mode == "decode":
             ops.rope_kv_write(q, k, v, H, KV, hd, self.inv_freq, self.position.rotary_dim,
                               ctx.row_seq, ctx.row_pos, ctx.new_len, table, k_pool, v_pool, rows_cap)
             out = ops.attention_decode(q, H, KV, hd, ctx.new_len, table, k_pool, v_pool, rows_cap,
                                        self.query_scale, self.softcap, self.window, ctx.dtype,
-                                       max_keys=ctx.max_rows_visible(site))
+                                       max_keys=ctx.max_rows_visible(site), **more)
+            if self.value_back is not None:
+                self._turn(ctx, out, H, self.value_back)
             return self._project_out(ctx, x, out)
         # Sequences that go on by several tokens (or some start while others go on) see cached positions and the
         # step's own rows.  The attention reads the cached ones where they lie, as earlier steps left them, and the
@@ -161,7 +222,9 @@ class Attention(Mixer):
                                     self.query_scale, self.softcap, self.window, ctx.dtype,
                                     row_seq=ctx.row_seq, row_pos=ctx.row_pos,
                                     cached=(ctx.new_len, table, k_pool, v_pool, rows_cap) if extend else None,
-                                    wide_weights=self.precise_weights)
+                                    wide_weights=self.precise_weights, **more)
+        if self.value_back is not None:
+            self._turn(ctx, out, H, self.value_back)
         if extend and owns_cache:
             row_seq, row_pos, new_len = ctx.row_seq, ctx.row_pos, ctx.new_len
             ctx.after_readers(lambda: ops.kv_write(k, v, KV, hd, row_seq, row_pos, new_len, table, k_pool, v_pool, rows_cap))

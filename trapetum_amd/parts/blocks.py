@@ -2,7 +2,7 @@
 
 sandwich  x += post_mixer_norm(mixer(pre_mixer_norm(x)));
           x += post_ff_norm(ff(pre_ff_norm(x)))          (runtime/src/lib.rs:4527-4540)
-pre_norm  x += mixer(pre_mixer_norm(x));  x += ff(pre_ff_norm(x))
+pre_norm  x += mixer(pre_mixer_norm(x));  x += ff(pre_ff_norm(x)); the feed-forward may be absent
           (the reference's other layer type, runtime/src/lib.rs:721-730)
 post_norm x += post_mixer_norm(mixer(c1(x)));  x += post_ff_norm(ff(c2(x))): no norm in front of a sub-layer; c1
           and c2 are what it reads of the stream, the stream itself or (input_conv) the stream through a short
@@ -69,6 +69,12 @@ class SandwichBlock(Block):
 
 
 class PreNormBlock(Block):
+    def __init__(self, mixer, feed_forward, make_norm):
+        self.mixer = mixer
+        self.feed_forward = feed_forward                 # None: the layer is its mixer behind its norm
+        sites = self.norm_sites() if feed_forward is not None else self.norm_sites()[:1]
+        self.norms = {name: make_norm(name) for name in sites}
+
     @classmethod
     def norm_sites(cls):
         return ("pre_mixer_norm", "pre_ff_norm")
@@ -82,6 +88,10 @@ class PreNormBlock(Block):
         ctx.dump("mixer_in", x)
         a = self.mixer.forward(ctx, x, site)
         ctx.dump("mixer_out", a)
+        if self.feed_forward is None:
+            normed_next = add_then_norm(ctx, stream, a, None, next_norm)
+            ctx.dump("layer_out", stream)
+            return stream, normed_next
         x = add_then_norm(ctx, stream, a, None, n["pre_ff_norm"])
         ctx.dump("after_mixer", stream)
         m = self.feed_forward.forward(ctx, x)

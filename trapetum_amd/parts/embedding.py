@@ -1,32 +1,42 @@
 """Token embedding and the head that turns rows into logits.
 
-Embedding: table[token] * scale in fp32 (the reference bakes Gemma's sqrt(hidden)
+Embedding: table[token] * scale in fp32, then (optionally) a norm of the row (the reference bakes Gemma's sqrt(hidden)
 into an fp16 table at export, model/export_gemma.py:59-61; here the table stays
 as stored so that a tied head can use it unscaled, :73).  Head: logits = rows @
 table^T with fp32 accumulation and fp32 output, then c * tanh(z / c) when a cap is
 set (runtime/src/lib.rs:4558-4560, on the host there; in the product's epilogue here).
 """
 from ..models.spec import TensorSpec
-from ..registry import register_part
+from ..registry import build_part, register_part
 from .base import Embedding, Head
 
 
 class ScaledEmbedding(Embedding):
-    def __init__(self, vocab_size, hidden_size, scale, tensor="weight"):
+    def __init__(self, vocab_size, hidden_size, scale, tensor="weight", norm=None):
+        """norm: (registered norm, parameters) applied to every embedded row, in fp32; its tensors stand beside the
+        table under the names its parameters give."""
         self.vocab_size = vocab_size
         self.hidden_size = hidden_size
         self.scale = float(scale)
         self.tensor = tensor             # the table's local name ("" when the prefix is the whole name)
+        self.norm = build_part("norm", norm) if norm is not None else None
 
     def tensor_specs(self):
-        return {self.tensor: TensorSpec((self.vocab_size, self.hidden_size), init="embedding")}
+        specs = {self.tensor: TensorSpec((self.vocab_size, self.hidden_size), init="embedding")}
+        if self.norm is not None:
+            specs.update(self.norm.tensor_specs())
+        return specs
 
     def bind(self, tensors, rt):
         self.rt = rt
         self.table = rt.matrix(tensors[self.tensor])
+        if self.norm is not None:
+            self.norm.bind({k: tensors[k] for k in self.norm.tensor_specs()}, rt)
 
     def forward(self, ctx, tokens):
-        return ctx.ops.embed_rows(tokens, self.table, self.scale)
+        import torch
+        rows = ctx.ops.embed_rows(tokens, self.table, self.scale)
+        return rows if self.norm is None else self.norm.forward(ctx, rows, torch.float32)
 
 
 class LinearHead(Head):

@@ -1,4 +1,5 @@
-"""Gated feed-forward: down(act(gate x) * up x).
+"""Gated feed-forward: down(act(gate x) * up x), or with a limit L and a shift c: g = min(gate x, L),
+u = clamp(up x, -L, L), down(act(g) * (u + c)).
 
 The reference computes gate and up as two fp32 vectors, applies
 0.5 g (1 + tanh(0.7978845608 (g + 0.044715 g^3))) * u in fp32 and rounds once
@@ -13,10 +14,13 @@ from .base import FeedForward
 
 class GatedMLP(FeedForward):
     def __init__(self, hidden_size, intermediate_size, activation,
-                 tensors=("gate_proj.weight", "up_proj.weight", "down_proj.weight")):
+                 tensors=("gate_proj.weight", "up_proj.weight", "down_proj.weight"), limit=None, up_shift=0.0):
+        """activation: gelu_tanh, silu, relu or quick_gelu (g sigmoid(1.702 g)).  limit None: no clamps."""
         self.hidden_size = hidden_size
         self.intermediate_size = intermediate_size
         self.activation = activation
+        self.limit = None if limit is None else float(limit)
+        self.up_shift = float(up_shift)
         self.names = tuple(tensors)      # local names of the gate, up and down matrices
 
     def tensor_specs(self):
@@ -32,7 +36,11 @@ class GatedMLP(FeedForward):
 
     def forward(self, ctx, x, out=None):
         """out: a contiguous float32 [M, hidden] to fill (a caller that adds this layer's output to another's)."""
-        act = ctx.ops.gated_linear(x, self.w_gate_up, self.intermediate_size, self.activation, ctx.dtype)
+        if self.limit is None and self.up_shift == 0.0:
+            act = ctx.ops.gated_linear(x, self.w_gate_up, self.intermediate_size, self.activation, ctx.dtype)
+        else:
+            act = ctx.ops.gated_linear(x, self.w_gate_up, self.intermediate_size, self.activation, ctx.dtype,
+                                       limit=self.limit, up_shift=self.up_shift)
         if out is not None:
             return ctx.ops.linear(act, self.w_down, out.dtype, out=out)
         return ctx.ops.linear(act, self.w_down, ctx.dtype, defer=True)

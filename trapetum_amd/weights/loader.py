@@ -52,8 +52,9 @@ def check_source(source, layout, folder="<memory>"):
     wrong_shape, wrong_dtype = [], []
     for name in sorted(need & have):
         ts = layout[name]
-        if tuple(source.shape(name)) != tuple(ts.shape):
-            wrong_shape.append((name, tuple(ts.shape), tuple(source.shape(name))))
+        found, free = tuple(source.shape(name)), set(getattr(ts, "free", ()))
+        if len(found) != len(ts.shape) or any(f != e for i, (f, e) in enumerate(zip(found, ts.shape)) if i not in free):
+            wrong_shape.append((name, tuple("any" if i in free else e for i, e in enumerate(ts.shape)), found))
         dt = source.dtype(name)
         if ts.dtype == "float" and dt not in _FLOATS:
             wrong_dtype.append((name, "a floating-point type", str(dt)))
