@@ -6,7 +6,9 @@
 // shapes the matrix-core kernels refuse.  Formula and order as the reference's attn_k
 // (runtime/cuda/codebook_gemv.cu:240-270): score = dot * scale, cap * tanh(score / cap), softmax, weighted
 // sum of v, kv head = head / (heads / kv_heads); the scale is an argument (rsqrt(head_dim) there), and a
-// window W hides keys with p - t >= W (none there).
+// window W hides keys with p - t >= W (none there).  Beyond the reference: with chunks of C positions the query at p
+// sees only keys from floor(p / C) C on; a head may have a temperature that multiplies its scores and a sink, a score
+// without key or value whose exponential joins the denominator once, after the keys.
 #include "common.h"
 
 struct AttnSimpleArgs {
@@ -20,6 +22,7 @@ struct AttnSimpleArgs {
     const int* new_len; const int* table; int table_w; const void* k_pool; const void* v_pool; int page; int rows_cap;
     void* out;
     int H, KV, hd; float scale, cap; int window; int paged;
+    int chunk; const float* head_scale; const float* sink;        // 0 and null: none
 };
 
 // NJ: elements of a head a lane holds (head sizes up to 64 NJ)
@@ -35,7 +38,9 @@ attn_simple_k(AttnSimpleArgs a) {
         p = a.row_pos[r];
         if (a.new_len) start = a.new_len[seq] - (a.cu_rows[seq + 1] - a.cu_rows[seq]);
     }
-    const int lo = a.window > 0 ? max(0, p - a.window + 1) : 0;
+    int lo = a.window > 0 ? max(0, p - a.window + 1) : 0;
+    if (a.chunk > 0) lo = max(lo, p / a.chunk * a.chunk);
+    const float scale = a.head_scale ? a.scale * a.head_scale[h] : a.scale;
     const T* q = (const T*)a.q + (size_t)r * a.q_stride + (size_t)h * a.hd;
     float qv[NJ], o[NJ];
 #pragma unroll
@@ -74,7 +79,7 @@ attn_simple_k(AttnSimpleArgs a) {
         float part = 0.f;
 #pragma unroll
         for (int j = 0; j < NJ; j++) part = fmaf(qv[j], kk[j], part);
-        float s = wave_sum(part) * a.scale;
+        float s = wave_sum(part) * scale;
         if (a.cap > 0.f) s = softcap_f(s, a.cap);
         const float m_new = fmaxf(m, s);
         const float alpha = expf(m - m_new), pr = expf(s - m_new);
@@ -95,6 +100,13 @@ attn_simple_k(AttnSimpleArgs a) {
         if (t + 2 > p) break;
         fetch(t + 4, k1, v1);
         use(k2, v2);
+    }
+    if (a.sink) {
+        const float sk = a.sink[h], m_new = fmaxf(m, sk);
+        const float alpha = expf(m - m_new);
+        l = l * alpha + expf(sk - m_new);
+#pragma unroll
+        for (int j = 0; j < NJ; j++) o[j] *= alpha;
     }
     T* out = (T*)a.out + ((size_t)r * a.H + h) * a.hd;
     const float inv = 1.f / l;
@@ -126,7 +138,9 @@ extern "C" int tp_attn_simple_prefill(const void* q, long q_stride, const void* 
                                       int dtype, int M, int H, int KV, int hd, const int* cu_rows, const int* row_seq,
                                       const int* row_pos, const int* new_len, const int* table, int table_w,
                                       const void* k_pool, const void* v_pool, int page, int rows_cap,
-                                      float scale, float cap, int window, void* out, void* stream) {
+                                      float scale, float cap, int window, int chunk, const float* head_scale, const float* sink,
+                                      void* out, void* stream) {
+    TP_REQUIRE(chunk >= 0, "attention: chunks of %d positions", chunk);
     TP_REQUIRE(!new_len || (table && k_pool && v_pool && page > 0 && table_w > 0), "attention: cached positions need the page table and the pools");
     AttnSimpleArgs a{};
     a.q = q; a.q_stride = q_stride; a.k = k; a.k_stride = k_stride; a.v = v; a.v_stride = v_stride;
@@ -134,17 +148,20 @@ extern "C" int tp_attn_simple_prefill(const void* q, long q_stride, const void* 
     a.new_len = new_len; a.table = table; a.table_w = table_w; a.k_pool = k_pool; a.v_pool = v_pool;
     a.page = new_len ? page : 1; a.rows_cap = new_len ? rows_cap : 0;
     a.out = out; a.H = H; a.KV = KV; a.hd = hd; a.scale = scale; a.cap = cap; a.window = window; a.paged = 0;
+    a.chunk = chunk; a.head_scale = head_scale; a.sink = sink;
     return launch(a, dtype, M, (hipStream_t)stream);
 }
 
 extern "C" int tp_attn_simple_decode(const void* q, long q_stride, int dtype, int n_seq, int H, int KV, int hd,
                                      const int* new_len, const int* table, int table_w, const void* k_pool,
                                      const void* v_pool, int page, int rows_cap, float scale, float cap, int window,
-                                     void* out, void* stream) {
+                                     int chunk, const float* head_scale, const float* sink, void* out, void* stream) {
+    TP_REQUIRE(chunk >= 0, "attention: chunks of %d positions", chunk);
     TP_REQUIRE(page > 0 && table_w > 0, "attention: page size %d, table width %d", page, table_w);
     AttnSimpleArgs a{};
     a.q = q; a.q_stride = q_stride; a.new_len = new_len; a.table = table; a.table_w = table_w;
     a.k_pool = k_pool; a.v_pool = v_pool; a.page = page; a.rows_cap = rows_cap;
     a.out = out; a.H = H; a.KV = KV; a.hd = hd; a.scale = scale; a.cap = cap; a.window = window; a.paged = 1;
+    a.chunk = chunk; a.head_scale = head_scale; a.sink = sink;
     return launch(a, dtype, n_seq, (hipStream_t)stream);
 }

@@ -89,7 +89,10 @@ __device__ __forceinline__ float gelu_tanh_fast(float g) {
 // bf16 products' epilogues take the two constants (`epi.x`, `epi.y`) and have no branch on the activation's kind.
 // ReLU is the limit of the form for c1 -> -infinity: with c1 = -1e30 the power of two is 0 for every g above 1e-28
 // and infinite for every g below -1e-28, so the quotient is g or -0 (and within 1e-28 of 0 in between).
-enum { TP_ACT_GELU_TANH = 0, TP_ACT_SILU = 1, TP_ACT_RELU = 2 };
+// A fourth, g sigmoid(1.702 g), is SiLU's form with c1 = -1.702 log2(e).  A gated product may also cut its sums first:
+// g' = min(g, limit), u' = clamp(u, -limit, limit), out = act(g') (u' + shift); limit = infinity and shift = 0 leave
+// the plain product act(g) u, bit for bit (`epi.z`, `epi.w`).
+enum { TP_ACT_GELU_TANH = 0, TP_ACT_SILU = 1, TP_ACT_RELU = 2, TP_ACT_QUICK_GELU = 3 };
 // which elements of a head a rotation pairs: (f, f + rotary_dim / 2) as the reference does
 // (runtime/cuda/codebook_gemv.cu:219-230), or neighbours (2f, 2f + 1)
 enum { TP_ROPE_HALVES = 0, TP_ROPE_NEIGHBOURS = 1 };
@@ -98,12 +101,25 @@ static inline bool tp_gate_constants(int act, float* c1, float* c3) {
     if (act == TP_ACT_GELU_TANH) { *c1 = -2.f * 0.7978845608f * LOG2E; *c3 = *c1 * 0.044715f; return true; }
     if (act == TP_ACT_SILU) { *c1 = -LOG2E; *c3 = 0.f; return true; }
     if (act == TP_ACT_RELU) { *c1 = -1e30f; *c3 = 0.f; return true; }
+    if (act == TP_ACT_QUICK_GELU) { *c1 = -1.702f * LOG2E; *c3 = 0.f; return true; }
     return false;
 }
-__device__ __forceinline__ float gate_act_fast(float g, float2 epi) {
+__device__ __forceinline__ float gate_act_fast(float g, float4 epi) {
     return g * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(g * __builtin_fmaf(epi.y, g * g, epi.x)));
+}
+// a gated product's output element from its gate and up sums
+__device__ __forceinline__ float gated_unit_fast(float g, float u, float4 epi) {
+    g = fminf(g, epi.z);
+    u = fminf(fmaxf(u, -epi.z), epi.z);
+    return gate_act_fast(g, epi) * (u + epi.w);
 }
 // the same in full float32 arithmetic, for the float32 path
 __device__ __forceinline__ float gate_act_exact(float g, int act) {
+    if (act == TP_ACT_QUICK_GELU) return g / (1.f + expf(-1.702f * g));
     return act == TP_ACT_SILU ? g / (1.f + expf(-g)) : (act == TP_ACT_RELU ? fmaxf(g, 0.f) : gelu_tanh_f(g));
+}
+__device__ __forceinline__ float gated_unit_exact(float g, float u, int act, float limit, float shift) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return gate_act_exact(g, act) * (u + shift);
 }

@@ -662,22 +662,22 @@ extern "C" int tp_scale_rows(float* x, long total, float scale, void* stream) {
 }
 
 template <typename T>
-__global__ void gated_act_k(const float* __restrict__ y, T* __restrict__ out, int I, int Ip2, int act) {
+__global__ void gated_act_k(const float* __restrict__ y, T* __restrict__ out, int I, int Ip2, int act, float limit, float shift) {
     const float* yr = y + (size_t)blockIdx.x * Ip2;
     T* orow = out + (size_t)blockIdx.x * I;
     for (int i = threadIdx.x; i < I; i += blockDim.x) {
         const int base = (i >> 4) * 32 + (i & 15);
-        st_f32(orow + i, gate_act_exact(yr[base], act) * yr[base + 16]);
+        st_f32(orow + i, gated_unit_exact(yr[base], yr[base + 16], act, limit, shift));
     }
 }
 
-extern "C" int tp_gated_act(const float* y, void* out, int dtype, int M, int I, int act, void* stream) {
+extern "C" int tp_gated_act(const float* y, void* out, int dtype, int M, int I, int act, float limit, float shift, void* stream) {
     TP_REQUIRE(M > 0 && I > 0, "gated_act: empty shape M=%d I=%d", M, I);
-    TP_REQUIRE(act == TP_ACT_GELU_TANH || act == TP_ACT_SILU || act == TP_ACT_RELU, "gated_act: unknown activation %d", act);
+    TP_REQUIRE(act == TP_ACT_GELU_TANH || act == TP_ACT_SILU || act == TP_ACT_RELU || act == TP_ACT_QUICK_GELU, "gated_act: unknown activation %d", act);
     const int Ip2 = 2 * ((I + 15) / 16) * 16;
     hipStream_t s = (hipStream_t)stream;
-    if (dtype == TP_BF16) gated_act_k<bf16_t><<<M, 256, 0, s>>>(y, (bf16_t*)out, I, Ip2, act);
-    else if (dtype == TP_F32) gated_act_k<float><<<M, 256, 0, s>>>(y, (float*)out, I, Ip2, act);
+    if (dtype == TP_BF16) gated_act_k<bf16_t><<<M, 256, 0, s>>>(y, (bf16_t*)out, I, Ip2, act, limit, shift);
+    else if (dtype == TP_F32) gated_act_k<float><<<M, 256, 0, s>>>(y, (float*)out, I, Ip2, act, limit, shift);
     else return tp_fail("gated_act: unknown dtype %d", dtype);
     return tp_check_launch("gated_act");
 }

@@ -14,6 +14,7 @@ struct GemmArgs {
     int epilogue; float cap;
     int units;              // gated: columns of the output (the feed-forward width)
     int act;                // gated: the gate's activation (TP_ACT_*)
+    float limit, shift;     // gated: the sums are cut at +-limit (infinity: not at all), the up sum gets `shift` added
     void* workspace; size_t workspace_bytes;
     int defer;              // split products: leave the K slices in the workspace [slices, M, N] for the consumer to add
     int algo;               // the caller's choice of kernel (0: none; see tp_linear)
@@ -21,8 +22,8 @@ struct GemmArgs {
 };
 
 // the constants a kernel's epilogue takes: the cap, or the gate activation's two
-static inline float2 epi_constants(const GemmArgs& a) {
-    float2 e = make_float2(a.cap, 0.f);
+static inline float4 epi_constants(const GemmArgs& a) {
+    float4 e = make_float4(a.cap, 0.f, a.limit, a.shift);
     if (a.epilogue == TP_EPI_GATED) tp_gate_constants(a.act, &e.x, &e.y);
     return e;
 }

@@ -38,7 +38,7 @@ __device__ __forceinline__ unsigned in_register(unsigned v) {
 // out in one store where the row length allows the alignment.
 template <int EPI, int TM, int TN>
 __device__ __forceinline__ void store_tile(const f32x4 (&acc)[TM][TN], void* __restrict__ Y, int M, int N, int m0, int n0,
-                                           int wm, int wn, int r, int g, int out_dtype, float2 epi, int units) {
+                                           int wm, int wn, int r, int g, int out_dtype, float4 epi, int units) {
     const int width = EPI == TP_EPI_GATED ? units : N;
     const bool wide = (width & 3) == 0;
 #pragma unroll
@@ -52,7 +52,7 @@ __device__ __forceinline__ void store_tile(const f32x4 (&acc)[TM][TN], void* __r
             if (EPI == TP_EPI_GATED) {
                 col = ((n0 + wn * 16 * TN + j * 16) >> 1) + g * 4;
 #pragma unroll
-                for (int v = 0; v < 4; v++) o[v] = gate_act_fast(acc[i][j][v], epi) * acc[i][j + 1 < TN ? j + 1 : j][v];
+                for (int v = 0; v < 4; v++) o[v] = gated_unit_fast(acc[i][j][v], acc[i][j + 1 < TN ? j + 1 : j][v], epi);
             } else {
                 col = n0 + wn * 16 * TN + j * 16 + g * 4;
 #pragma unroll
@@ -88,7 +88,7 @@ __device__ __forceinline__ void store_tile(const f32x4 (&acc)[TM][TN], void* __r
 template <int EPI, int TM, int TN, bool SHORT, int KS = BK, int WM = 2, bool DEEP = false>
 __global__ void __launch_bounds__(256, 2)
 gemm_mfma_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __restrict__ Y,
-            int M, int N, int K, int m_tiles, int out_dtype, float2 epi, int units, int k_per_split, int xcd_panels) {
+            int M, int N, int K, int m_tiles, int out_dtype, float4 epi, int units, int k_per_split, int xcd_panels) {
     constexpr int WN = 4 / WM, BM = 16 * WM * TM, BN = 16 * WN * TN, BK = KS, LDS = KS, CPR = KS / 8;
     constexpr int LA = BM * KS / 2048, LB = BN * KS / 2048;    // 16-byte chunks of a step's tile per thread
     static_assert(BM * KS % 2048 == 0 && BN * KS % 2048 == 0, "a step's tile is a whole number of chunks per thread");
@@ -233,7 +233,7 @@ gemm_mfma_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __
 template <int EPI, int TN>
 __global__ void __launch_bounds__(256, 2)
 gemm_mfma_direct_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __restrict__ Y,
-                   int M, int N, int K, int m_tiles, int out_dtype, float2 epi, int units, int k_per_split, int xcd_panels) {
+                   int M, int N, int K, int m_tiles, int out_dtype, float4 epi, int units, int k_per_split, int xcd_panels) {
     constexpr int TM = 4, BM = 128, BN = 32 * TN, LDS = BK;
     __shared__ __attribute__((aligned(16))) bf16_t As[BM * LDS];
     __shared__ __attribute__((aligned(16))) bf16_t Bs[BN * LDS];

@@ -27,7 +27,7 @@ union Frag8 { uint4 u; bf16x8 v; };
 template <int NG, int NS>
 __global__ void __launch_bounds__(256)
 gemm_rows8_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __restrict__ Y, float* __restrict__ part,
-             int M, int N, int K, int k_per_split, int n_splits, int out_dtype, int epilogue, float2 epi, int units) {
+             int M, int N, int K, int k_per_split, int n_splits, int out_dtype, int epilogue, float4 epi, int units) {
     __shared__ float red[4][NG][64][4];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r = lane & 7, piece = lane >> 3;
     const int split = blockIdx.y;
@@ -111,7 +111,7 @@ gemm_rows8_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* _
         for (int p = 0; p < NG / 2; p++) {
             const int unit = blockIdx.x * (NG * 4) + p * 8 + wr;
             if (unit >= units) continue;
-            const float o = gate_act_fast(v[p], epi) * v[p + NG / 2];
+            const float o = gated_unit_fast(v[p], v[p + NG / 2], epi);
             if (out_dtype == TP_F32) ((float*)Y)[(size_t)m * units + unit] = o;
             else ((bf16_t*)Y)[(size_t)m * units + unit] = f32_to_bf16(o);
         }

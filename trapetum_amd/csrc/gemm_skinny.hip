@@ -33,7 +33,7 @@ __device__ __forceinline__ void store_out(void* y, int out_dtype, size_t idx, fl
 template <int MT, int NT>
 __global__ void __launch_bounds__(256)
 gemm_skinny_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __restrict__ Y, float* __restrict__ part,
-              int M, int N, int K, int k_per_split, int n_splits, int out_dtype, int epilogue, float2 epi, int units) {
+              int M, int N, int K, int k_per_split, int n_splits, int out_dtype, int epilogue, float4 epi, int units) {
     __shared__ float red[4][MT][64][4];                   // one W tile's partial tiles of the four waves at a time
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
     const int n0 = blockIdx.x * (16 * NT);
@@ -148,7 +148,7 @@ gemm_skinny_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* 
 #pragma unroll
             for (int s = 0; s + 1 < NT; s += 2) {         // tiles alternate: 16 gate rows, the 16 up rows of the same units
                 const int unit = ((n0 + s * 16) >> 1) + nl;
-                if (unit < units) store_out(Y, out_dtype, (size_t)m * units + unit, gate_act_fast(v[t][s], epi) * v[t][s + 1]);
+                if (unit < units) store_out(Y, out_dtype, (size_t)m * units + unit, gated_unit_fast(v[t][s], v[t][s + 1], epi));
             }
         } else {
 #pragma unroll
@@ -165,7 +165,7 @@ gemm_skinny_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* 
 
 // adds the K slices in slice order and applies the epilogue
 __global__ void skinny_reduce_k(const float* __restrict__ part, void* __restrict__ Y, int M, int N, int n_splits,
-                                int out_dtype, int epilogue, float2 epi, int units) {
+                                int out_dtype, int epilogue, float4 epi, int units) {
     const int cols = epilogue == TP_EPI_GATED ? units : N;
     const long total = (long)M * cols;
     for (long idx = blockIdx.x * (long)blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
@@ -178,7 +178,7 @@ __global__ void skinny_reduce_k(const float* __restrict__ part, void* __restrict
                 gsum += p[ng];
                 usum += p[ng + 16];
             }
-            store_out(Y, out_dtype, idx, gate_act_fast(gsum, epi) * usum);
+            store_out(Y, out_dtype, idx, gated_unit_fast(gsum, usum, epi));
         } else {
             float sum = 0.f;
             for (int s = 0; s < n_splits; s++) sum += part[((size_t)s * M + m) * N + c];

@@ -33,11 +33,17 @@ _CORE_SIGS = {
     "tp_sum_slices": [_P, _I, _L, _P, _I, _L, _P],
     "tp_rope_kv_write": [_P, _L, _P, _L, _P, _L, _I, _I, _I, _I, _I, _P, _I, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _P],
     "tp_kv_write": [_P, _L, _P, _L, _I, _I, _I, _I, _P, _P, _P, _P, _I, _P, _P, _I, _I, _P],
-    "tp_gated_act": [_P, _P, _I, _I, _I, _I, _P],
-    "tp_linear": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P, _L, _I, _I, _P],
+    "tp_gated_act": [_P, _P, _I, _I, _I, _I, _F, _F, _P],
+    "tp_linear": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _F, _F, _P, _L, _I, _I, _P],
+    "tp_shift_mix": [_P, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
+    "tp_unary_tanh": [_P, _I, _L, _P],
+    "tp_weighted_sum": [_P, _F, _P, _F, _I, _P, _L, _P],
+    "tp_head_norm_gate": [_P, _P, _P, _L, _I, _F, _P, _I, _I, _I, _I, _I, _P],
+    "tp_time_mix_scan": [_P, _L, _P, _L, _P, _L, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _P],
+    "tp_matrix_memory_scan": [_P, _L, _P, _L, _P, _L, _I, _P, _F, _F, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
     "tp_linear_workspace_bytes": [_I, _I, _I, _I, _I, _I, _I, _I, _I],
-    "tp_attn_simple_prefill": [_P, _L, _P, _L, _P, _L, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _F, _F, _I, _P, _P],
-    "tp_attn_simple_decode": [_P, _L, _I, _I, _I, _I, _I, _P, _P, _I, _P, _P, _I, _I, _F, _F, _I, _P, _P],
+    "tp_attn_simple_prefill": [_P, _L, _P, _L, _P, _L, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _F, _F, _I, _I, _P, _P, _P, _P],
+    "tp_attn_simple_decode": [_P, _L, _I, _I, _I, _I, _I, _P, _P, _I, _P, _P, _I, _I, _F, _F, _I, _I, _P, _P, _P, _P],
     "tp_argmax": [_P, _I, _I, _P, _P, _P],
     "tp_argmax_workspace_bytes": [_I, _I],
     "tp_repetition_penalty": [_P, _I, _I, _P, _I, _F, _P],
@@ -58,7 +64,8 @@ _ATTN_SIGS = {
 
 EPI_NONE, EPI_SOFTCAP, EPI_GATED = 0, 1, 2
 ROPE_PAIRINGS = {"halves": 0, "neighbours": 1}          # the kernel library's TP_ROPE_* enumerators
-GATE_ACTIVATIONS = {"gelu_tanh": 0, "silu": 1, "relu": 2}       # what a gated product's epilogue can apply to the gate
+GATE_ACTIVATIONS = {"gelu_tanh": 0, "silu": 1, "relu": 2, "quick_gelu": 3}       # what a gated product's epilogue can apply to the gate
+HEAD_GATES = {"sigmoid": 0, "silu": 1}               # what `head_norm_gate` multiplies a normed head by: act(g)
 ROUTE_SCORES = {"softmax": 0, "sigmoid": 1}          # how a router's logits become scores
 CONV_ACTIVATIONS = {None: 0, "silu": 1}
 GATE_GROUP = 16
@@ -458,6 +465,129 @@ class HipOps:
                    int(max_count), heads, groups, n_state, head_dim, chunk, ws.data_ptr() if ws is not None else None, nbytes, self._stream())
         return y
 
+    # ---- mixers that carry a matrix per head from token to token --------------------------------------------------------
+    def _geometry(self, what, m, slot_ids, cu_rows, row_seq=None):
+        n_seq = cu_rows.numel() - 1
+        for t, n in ((cu_rows, n_seq + 1), (slot_ids, n_seq)) + (((row_seq, m),) if row_seq is not None else ()):
+            if t.dtype != torch.int32 or t.numel() != n:
+                raise KernelError(f"{what}: cu_rows, row_seq and slot_ids must be int32 of the step's geometry")
+        return n_seq
+
+    def shift_mix(self, x, mu, state, slot_ids, cu_rows, row_seq, one_row_each=False):
+        """out[s, r] = x[r] + (x[r - 1] - x[r]) * mu[s] within each sequence; the row before a sequence's first row of
+        the step is state[slot] (float32 [slots, D]), which then takes the sequence's last row.  mu float32 [S, D];
+        returns [S, M, D] of x's dtype."""
+        self._dev(x, mu, state, slot_ids, cu_rows, row_seq)
+        if x.dim() != 2 or not x.is_contiguous():
+            raise KernelError("shift_mix: rows must be a contiguous matrix")
+        m, d = x.shape
+        if mu.dtype != torch.float32 or mu.dim() != 2 or mu.shape[1] != d or not mu.is_contiguous():
+            raise KernelError(f"shift_mix: the mixing vectors must be contiguous float32 [mixes, {d}]")
+        if state.dtype != torch.float32 or state.dim() != 2 or state.shape[1] != d or not state.is_contiguous():
+            raise KernelError(f"shift_mix: the state must be contiguous float32 [slots, {d}]")
+        n_seq = self._geometry("shift_mix", m, slot_ids, cu_rows, row_seq)
+        out = torch.empty((mu.shape[0], m, d), dtype=x.dtype, device=self.device)
+        self._call(self.lib, "tp_shift_mix", x.data_ptr(), _code(x.dtype), mu.data_ptr(), mu.shape[0], state.data_ptr(), slot_ids.data_ptr(),
+                   cu_rows.data_ptr(), row_seq.data_ptr(), out.data_ptr(), m, n_seq, d, 1 if one_row_each else 0, self._stream())
+        return out
+
+    def unary_(self, x, name):
+        """In place on a contiguous tensor: x <- tanh(x)."""
+        if name != "tanh":
+            raise KernelError(f"unary_: '{name}' has no kernel (tanh)")
+        self._dev(x)
+        if not x.is_contiguous():
+            raise KernelError("unary_: expected a contiguous tensor")
+        self._call(self.lib, "tp_unary_tanh", x.data_ptr(), _code(x.dtype), x.numel(), self._stream())
+        return x
+
+    def weighted_sum(self, a, wa, b, wb):
+        """float32: wa * a + wb * b, for two contiguous tensors of one shape and dtype."""
+        self._dev(a, b)
+        if a.shape != b.shape or a.dtype != b.dtype or not a.is_contiguous() or not b.is_contiguous():
+            raise KernelError("weighted_sum: two contiguous tensors of one shape and dtype")
+        out = torch.empty(a.shape, dtype=torch.float32, device=self.device)
+        self._call(self.lib, "tp_weighted_sum", a.data_ptr(), float(wa), b.data_ptr(), float(wb), _code(a.dtype), out.data_ptr(), a.numel(), self._stream())
+        return out
+
+    def head_norm_gate(self, y, gain, g, eps, heads, activation, out_dtype):
+        """Every head's part of a row of y (float32 [M, D]) over its root mean square, times gain (float32 [D]), times
+        act(g) with act one of HEAD_GATES; g [M, D] of the output's dtype, possibly a view of wider rows."""
+        if activation not in HEAD_GATES:
+            raise KernelError(f"head_norm_gate: gate '{activation}' has no kernel ({', '.join(HEAD_GATES)})")
+        self._dev(y, gain, g)
+        if y.dtype != torch.float32 or y.dim() != 2 or not y.is_contiguous():
+            raise KernelError("head_norm_gate: rows must be a contiguous float32 matrix")
+        m, d = y.shape
+        if heads < 1 or d % heads:
+            raise KernelError(f"head_norm_gate: rows of {d} elements are not {heads} equal heads")
+        if gain.dtype != torch.float32 or gain.numel() != d or not gain.is_contiguous():
+            raise KernelError(f"head_norm_gate: the gain must be contiguous float32 [{d}]")
+        gs = self._rows(g, "head_norm_gate gates")
+        if tuple(g.shape) != (m, d) or g.dtype != out_dtype:
+            raise KernelError(f"head_norm_gate: gates must be {(m, d)} of the output's dtype {out_dtype}")
+        out = torch.empty((m, d), dtype=out_dtype, device=self.device)
+        self._call(self.lib, "tp_head_norm_gate", y.data_ptr(), gain.data_ptr(), g.data_ptr(), gs, _code(g.dtype), float(eps), out.data_ptr(),
+                   _code(out_dtype), m, heads, d // heads, HEAD_GATES[activation], self._stream())
+        return out
+
+    MAX_SCAN_DIM = 256             # key rows a lane of a scan keeps of its column, and columns of a block
+
+    def time_mix_scan(self, r, k, v, log_rate, w0, bonus, state, slot_ids, cu_rows, max_count, heads, dim):
+        """o = (S + diag(bonus) k v^T)^T r, then S <- diag(w) S + k v^T with w = exp(-exp(log_rate + w0)), row after row
+        of every sequence from state[slot] (float32 [slots, heads, dim, dim]: key row, value column), which is left
+        updated.  r, k, v [M, heads dim], possibly views of wider rows; log_rate float32 [M, heads dim]; w0 float32
+        [heads dim]; bonus float32 [heads, dim].  Returns float32 [M, heads dim]."""
+        self._dev(r, k, v, log_rate, w0, bonus, state, slot_ids, cu_rows)
+        m, inner = r.shape[0], heads * dim
+        rs, ks, vs = self._rows(r, "time_mix_scan r"), self._rows(k, "time_mix_scan k"), self._rows(v, "time_mix_scan v")
+        if any(tuple(t.shape) != (m, inner) for t in (r, k, v)) or not (r.dtype == k.dtype == v.dtype):
+            raise KernelError(f"time_mix_scan: r, k and v must be {(m, inner)} of one dtype")
+        if dim > self.MAX_SCAN_DIM:
+            raise KernelError(f"time_mix_scan: heads of {dim} channels exceed {self.MAX_SCAN_DIM}")
+        if log_rate.dtype != torch.float32 or tuple(log_rate.shape) != (m, inner) or not log_rate.is_contiguous():
+            raise KernelError(f"time_mix_scan: the decays' logarithms must be contiguous float32 {(m, inner)}")
+        for t in (w0, bonus):
+            if t.dtype != torch.float32 or t.numel() != inner or not t.is_contiguous():
+                raise KernelError(f"time_mix_scan: w0 and the bonus must be contiguous float32 of {inner} elements")
+        if state.dtype != torch.float32 or state.dim() != 4 or tuple(state.shape[1:]) != (heads, dim, dim) or not state.is_contiguous():
+            raise KernelError(f"time_mix_scan: the state must be contiguous float32 [slots, {heads}, {dim}, {dim}]")
+        n_seq = self._geometry("time_mix_scan", m, slot_ids, cu_rows)
+        y = torch.empty((m, inner), dtype=torch.float32, device=self.device)
+        self._call(self.lib, "tp_time_mix_scan", r.data_ptr(), rs, k.data_ptr(), ks, v.data_ptr(), vs, _code(r.dtype), log_rate.data_ptr(),
+                   w0.data_ptr(), bonus.data_ptr(), state.data_ptr(), slot_ids.data_ptr(), cu_rows.data_ptr(), y.data_ptr(), n_seq, heads, dim,
+                   self._stream())
+        return y
+
+    def matrix_memory_scan(self, q, k, v, gates, cap, q_scale, memory, normalizer, maximum, slot_ids, cu_rows, max_count, heads, dk, dv):
+        """gates float32 [M, 2 heads]: the input gates' sums, then the forget gates'.  i = cap tanh(. / cap),
+        f = logsigmoid(cap tanh(. / cap)), m' = max(f + m, i), S <- e^(f + m - m') S + e^(i - m') k v^T, n likewise with k,
+        o = S^T q' / (max(|n . q'|, e^(-m')) + 1e-6) with q' = q q_scale, row after row of every sequence from the states
+        memory [slots, heads, dk, dv], normalizer [slots, heads, dk] and maximum [slots, heads] (float32), which are left
+        updated.  q, k [M, heads dk] and v [M, heads dv] may be views of wider rows.  Returns float32 [M, heads dv]."""
+        self._dev(q, k, v, gates, memory, normalizer, maximum, slot_ids, cu_rows)
+        m = q.shape[0]
+        qs, ks, vs = self._rows(q, "matrix_memory_scan q"), self._rows(k, "matrix_memory_scan k"), self._rows(v, "matrix_memory_scan v")
+        if tuple(q.shape) != (m, heads * dk) or tuple(k.shape) != (m, heads * dk) or tuple(v.shape) != (m, heads * dv) or not (q.dtype == k.dtype == v.dtype):
+            raise KernelError(f"matrix_memory_scan: q, k {(m, heads * dk)} and v {(m, heads * dv)} of one dtype")
+        if dk > self.MAX_SCAN_DIM or dv > self.MAX_SCAN_DIM:
+            raise KernelError(f"matrix_memory_scan: heads of {dk} x {dv} exceed {self.MAX_SCAN_DIM}")
+        if gates.dtype != torch.float32 or tuple(gates.shape) != (m, 2 * heads) or not gates.is_contiguous():
+            raise KernelError(f"matrix_memory_scan: the gates' sums must be contiguous float32 {(m, 2 * heads)}")
+        for t, shape in ((memory, (heads, dk, dv)), (normalizer, (heads, dk)), (maximum, (heads,))):
+            if t.dtype != torch.float32 or tuple(t.shape[1:]) != shape or not t.is_contiguous():
+                raise KernelError(f"matrix_memory_scan: a state must be contiguous float32 [slots, {', '.join(map(str, shape))}]")
+        if not (memory.shape[0] == normalizer.shape[0] == maximum.shape[0]):
+            raise KernelError("matrix_memory_scan: the three states must have the same slots")
+        if not cap > 0:
+            raise KernelError("matrix_memory_scan: the gates' cap must be positive")
+        n_seq = self._geometry("matrix_memory_scan", m, slot_ids, cu_rows)
+        y = torch.empty((m, heads * dv), dtype=torch.float32, device=self.device)
+        self._call(self.lib, "tp_matrix_memory_scan", q.data_ptr(), qs, k.data_ptr(), ks, v.data_ptr(), vs, _code(q.dtype), gates.data_ptr(),
+                   float(cap), float(q_scale), memory.data_ptr(), normalizer.data_ptr(), maximum.data_ptr(), slot_ids.data_ptr(),
+                   cu_rows.data_ptr(), y.data_ptr(), n_seq, heads, dk, dv, self._stream())
+        return y
+
     def pair_norm_mean(self, a, b, gain_a, gain_b, eps):
         """float32 [M, D]: 0.5 (a / rms(a) * gain_a + b / rms(b) * gain_b), each row over its own root mean square."""
         self._dev(a, b, gain_a, gain_b)
@@ -558,7 +688,7 @@ class HipOps:
                    v_pool.data_ptr(), k_pool.shape[2], rows_cap, self._stream())
 
     # ---- matrix products -----------------------------------------------------------------------------
-    def _linear(self, x, w, out_dtype, epilogue, cap, units, defer=False, act=0, out=None):
+    def _linear(self, x, w, out_dtype, epilogue, cap, units, defer=False, act=0, out=None, limit=float("inf"), shift=0.0):
         self._dev(x, w)
         if x.dim() != 2 or w.dim() != 2 or not x.is_contiguous() or not w.is_contiguous():
             raise KernelError("linear: rows and matrix must be contiguous 2-D tensors")
@@ -575,7 +705,7 @@ class HipOps:
         if defer and epilogue == EPI_NONE and nbytes and nbytes % (m * n * 4) == 0 and nbytes // (m * n * 4) > 1:
             slices = torch.empty((nbytes // (m * n * 4), m, n), dtype=torch.float32, device=self.device)
             self._call(self.lib, "tp_linear", x.data_ptr(), w.data_ptr(), None, _code(x.dtype), _code(out_dtype),
-                       m, n, k, epilogue, float(cap), units, act, slices.data_ptr(), nbytes, 1, algo, self._stream())
+                       m, n, k, epilogue, float(cap), units, act, float(limit), float(shift), slices.data_ptr(), nbytes, 1, algo, self._stream())
             return SplitRows(slices)
         if out is None:
             out = torch.empty((m, cols), dtype=out_dtype, device=self.device)
@@ -584,8 +714,8 @@ class HipOps:
         self._dev(out)
         ws = torch.empty(nbytes, dtype=torch.uint8, device=self.device) if nbytes else None
         self._call(self.lib, "tp_linear", x.data_ptr(), w.data_ptr(), out.data_ptr(), _code(x.dtype), _code(out_dtype),
-                   m, n, k, epilogue, float(cap), units, act, ws.data_ptr() if ws is not None else None, nbytes, 0, algo,
-                   self._stream())
+                   m, n, k, epilogue, float(cap), units, act, float(limit), float(shift),
+                   ws.data_ptr() if ws is not None else None, nbytes, 0, algo, self._stream())
         return out
 
     def linear(self, x, w, out_dtype, softcap=None, defer=False, bias=None, out=None):
@@ -610,11 +740,16 @@ class HipOps:
             return self._linear(x, w, out_dtype, EPI_SOFTCAP, softcap, 0)
         return self._linear(x, w, out_dtype, EPI_NONE, 0.0, 0, defer=defer)
 
-    def gated_linear(self, x, w_packed, inter, activation, out_dtype):
-        """act(x @ gate^T) * (x @ up^T) over the packed matrix of `pack_gate_up`; activation: one of GATE_ACTIVATIONS."""
+    def gated_linear(self, x, w_packed, inter, activation, out_dtype, limit=None, up_shift=0.0):
+        """act(g) * (u + up_shift) with g = x @ gate^T and u = x @ up^T over the packed matrix of `pack_gate_up`;
+        activation: one of GATE_ACTIVATIONS.  limit: g is cut at it from above and u from both sides, before the
+        activation (None: neither is cut)."""
         if activation not in GATE_ACTIVATIONS:
             raise KernelError(f"gated_linear: activation '{activation}' has no kernel ({', '.join(GATE_ACTIVATIONS)})")
-        return self._linear(x, w_packed, out_dtype, EPI_GATED, 0.0, inter, act=GATE_ACTIVATIONS[activation])
+        if limit is not None and not limit > 0:
+            raise KernelError(f"gated_linear: the sums' limit must be positive, found {limit}")
+        return self._linear(x, w_packed, out_dtype, EPI_GATED, 0.0, inter, act=GATE_ACTIVATIONS[activation],
+                            limit=float("inf") if limit is None else limit, shift=up_shift)
 
     # ---- attention -------------------------------------------------------------------------------------
     DECODE_GROUP = 16              # query heads per kv head the matrix-core decode kernel takes
@@ -626,15 +761,19 @@ class HipOps:
             (not decode or H // KV <= self.DECODE_GROUP)
 
     def attention_prefill(self, q, k, v, H, KV, hd, cu_rows, max_count, scale, softcap, window, out_dtype,
-                          row_seq=None, row_pos=None, cached=None, shape=0, wide_weights=False):
+                          row_seq=None, row_pos=None, cached=None, shape=0, wide_weights=False, chunk=0, head_scale=None, sink=None):
         """Causal attention of the step's queries over the step's own rows of keys and values and, with
         `cached` = (new_len, table, k_pool, v_pool, rows_cap), over the positions before them, read in place from the
         cache as earlier steps left it (the step's own rows are not looked for there).  Without `cached` every sequence
         starts at position 0; with it row_pos holds absolute positions, sequence s's first row standing at
         new_len[s] - its count.  shape: the matrix-core kernel's block shape (0: chosen by the size of the step).
         wide_weights: the matrix-core kernel multiplies the values by softmax weights of 16 bits of mantissa (two bf16
-        terms) instead of 8; the plain kernel's weights are float32 in any case."""
-        self._dev(q, k, v, cu_rows)
+        terms) instead of 8; the plain kernel's weights are float32 in any case.
+        chunk C: a query at position p sees keys from floor(p / C) C on only.  head_scale, sink: float32 [H], a factor on
+        every head's scores and a score without key or value in every head's softmax.  With any of the three the step
+        runs on the plain kernel (the matrix-core kernels have none of them)."""
+        self._dev(q, k, v, cu_rows, head_scale, sink)
+        plain_only = self._head_vectors("attention_prefill", H, chunk, head_scale, sink)
         m = q.shape[0]
         qs, ks, vs = self._rows(q, "attention q"), self._rows(k, "attention k"), self._rows(v, "attention v")
         if q.shape[1] != H * hd or k.shape != (m, KV * hd) or v.shape != (m, KV * hd):
@@ -651,7 +790,7 @@ class HipOps:
             page, table_w, rows_cap = k_pool.shape[2], table.shape[1], rows_cap or 0
         ptr = lambda t: t.data_ptr() if t is not None else None
         out = torch.empty((m, H * hd), dtype=out_dtype, device=self.device)
-        if self._fast_attention(q.dtype, H, KV, hd, decode=False) and (cached is None or (page >= 16 and page & (page - 1) == 0)):
+        if not plain_only and self._fast_attention(q.dtype, H, KV, hd, decode=False) and (cached is None or (page >= 16 and page & (page - 1) == 0)):
             lib = self.attn_lib(hd, wide=wide_weights)
             self._call(lib, "tp_attn_prefill", q.data_ptr(), qs, k.data_ptr(), ks, v.data_ptr(), vs,
                        m, H, KV, cu_rows.data_ptr(), n_seq, int(max_count), ptr(new_len), ptr(table), table_w,
@@ -667,8 +806,17 @@ class HipOps:
         self._call(self.lib, "tp_attn_simple_prefill", q.data_ptr(), qs, k.data_ptr(), ks, v.data_ptr(), vs, _code(q.dtype),
                    m, H, KV, hd, cu_rows.data_ptr(), row_seq.data_ptr(), row_pos.data_ptr(), ptr(new_len), ptr(table), table_w,
                    ptr(k_pool), ptr(v_pool), page, rows_cap, float(scale), float(softcap),
-                   int(window), out.data_ptr(), self._stream())
+                   int(window), int(chunk), ptr(head_scale), ptr(sink), out.data_ptr(), self._stream())
         return out
+
+    def _head_vectors(self, what, H, chunk, head_scale, sink):
+        """Checks what only the plain attention kernel takes; whether any of it is asked for."""
+        if chunk < 0:
+            raise KernelError(f"{what}: chunks of {chunk} positions")
+        for t, name in ((head_scale, "head_scale"), (sink, "sink")):
+            if t is not None and (t.dtype != torch.float32 or t.numel() != H or not t.is_contiguous()):
+                raise KernelError(f"{what}: {name} must be contiguous float32 [{H}]")
+        return bool(chunk) or head_scale is not None or sink is not None
 
     @staticmethod
     def decode_splits(n, KV, hd, keys):
@@ -690,11 +838,13 @@ class HipOps:
             raise KernelError(f"{what}: the page table must be contiguous int32 [sequences, pages]")
 
     def attention_decode(self, q, H, KV, hd, new_len, table, k_pool, v_pool, rows_cap, scale, softcap, window,
-                         out_dtype, max_keys=None, splits=None, head_groups=None):
+                         out_dtype, max_keys=None, splits=None, head_groups=None, chunk=0, head_scale=None, sink=None):
         """head_groups: cut the query heads into that many groups (a multiple of KV), each read the pool head
         `group % KV` by a block of its own: for caches whose one kv head serves many heads, where one block would
-        otherwise form all their weighted sums.  The plain kernel takes any grouping as it is."""
-        self._dev(q, new_len, table, k_pool, v_pool)
+        otherwise form all their weighted sums.  The plain kernel takes any grouping as it is.
+        chunk, head_scale, sink: as in `attention_prefill`."""
+        self._dev(q, new_len, table, k_pool, v_pool, head_scale, sink)
+        plain_only = self._head_vectors("attention_decode", H, chunk, head_scale, sink)
         n = q.shape[0]
         qs = self._rows(q, "attention q")
         if q.shape[1] != H * hd:
@@ -705,7 +855,7 @@ class HipOps:
         groups = int(head_groups) if head_groups else KV
         if groups % KV or H % groups:
             raise KernelError(f"attention_decode: {H} heads in {groups} groups on {KV} kv heads")
-        if self._fast_attention(q.dtype, H, groups, hd) and page >= 16 and page & (page - 1) == 0:
+        if not plain_only and self._fast_attention(q.dtype, H, groups, hd) and page >= 16 and page & (page - 1) == 0:
             lib = self.attn_lib(hd)
             keys = int(max_keys) if max_keys else k_pool.shape[0] * k_pool.shape[2]
             nsplit = int(splits) if splits else self.decode_splits(n, groups, hd, keys)
@@ -724,7 +874,8 @@ class HipOps:
             return out
         self._call(self.lib, "tp_attn_simple_decode", q.data_ptr(), qs, _code(q.dtype), n, H, KV, hd, new_len.data_ptr(),
                    table.data_ptr(), table.shape[1], k_pool.data_ptr(), v_pool.data_ptr(), k_pool.shape[2], rows_cap,
-                   float(scale), float(softcap), int(window), out.data_ptr(), self._stream())
+                   float(scale), float(softcap), int(window), int(chunk), head_scale.data_ptr() if head_scale is not None else None,
+                   sink.data_ptr() if sink is not None else None, out.data_ptr(), self._stream())
         return out
 
     def fuses_decode_step(self, dtype, H, KV, hd, k_pool):
