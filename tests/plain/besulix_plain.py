@@ -182,5 +182,15 @@ def forward(cfg, w, tokens, layers_out=None):
             layers_out.append(x.clone())
     x = unit_rms(x, eps) * w["final.norm"]
     z = x @ w["head"].T
-    cap = cfg["logit_softcap"]
-    return cap * torch.tanh(z / cap)
+    cap = cfg.get("logit_softcap")
+    return z if cap is None else cap * torch.tanh(z / cap)
+
+
+def greedy_generate(cfg, w, prompt, n):
+    toks, out = list(prompt), []
+    for _ in range(n):
+        z = forward(cfg, w, toks)[-1]
+        tok = int(torch.nonzero(z == z.max())[0])
+        out.append(tok)
+        toks.append(tok)
+    return out
