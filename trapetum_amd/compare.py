@@ -1,6 +1,7 @@
-"""Two designs side by side at equal layer sizes: Golepel or Lutovik next to Gemma-2, random weights, one MI355X.
+"""Two designs side by side at equal layer sizes: Golepel or Lutovik next to Gemma-2, Besulix next to Lutovik, random
+weights, one MI355X.
 
-    python bench.py --compare golepel|lutovik [--sizes 2b|9b] [--layers L] [--steps K] [--warmup W]
+    python bench.py --compare golepel|lutovik|besulix [--sizes 2b|9b] [--layers L] [--steps K] [--warmup W]
 
 For each design: tokens per second of a prefill of 2,048 tokens and of the generation loop's decode steps at batch 8
 and 1 (HIP graphs, greedy choice on the device), and the time of the kernels a step spends its time in, one by one at
@@ -16,6 +17,10 @@ layers with a dense feed-forward, the second runs an attention (keys of 128, val
 mixer (heads of 64 channels filling the width, a state of 128 rows, 4 groups, 4 taps), and the third is an attention
 layer on the first one's cache; the second and third have 8 experts of half the dense width, 2 chosen, and a shared
 expert of a quarter of it (`time_lutovik_kernels`).
+The Besulix sizes: the same width, vocabulary and number of layers; layers alternate between a parallel layer with a
+dense feed-forward of Gemma's width (left: 16 heads on 4 kv heads of 128, values of 128, a rotation of 64 elements,
+chunks of 1,024 positions; right: time-mixing heads of 64 channels filling the width) and a matrix-memory layer without
+a feed-forward (heads of 128 key and 256 value elements filling the width) (`time_besulix_kernels`).
 """
 import json
 import sys
@@ -64,6 +69,20 @@ def lutovik_config(which, layers=0):
             out.append({"type": "attention", "mixer": att, "mlp": {"kind": "dense", "ff": I}})
     return LutovikConfig.from_dict({"architecture": "Lutovik", "vocab": g["vocab_size"], "width": D, "embedding": {"scale": D ** 0.5},
                                     "norm": {"eps": 1e-6}, "layers": out})
+
+
+def besulix_config(which, layers=0):
+    from .config import BesulixConfig
+    g = dict(SIZES, **OTHER_SIZES[which])
+    n = layers or g["num_hidden_layers"]
+    D, I = g["hidden_size"], g["intermediate_size"]
+    left = {"heads": 16, "kv_heads": 4, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "rot": {"base": 250000.0, "dims": 64},
+            "mask": {"size": 1024}}
+    par = {"type": "parallel", "mixer": {"left": left, "left_scale": 0.8, "right": {"heads": D // 64, "dim": 64}, "right_scale": 0.9},
+           "mlp": {"kind": "dense", "ff": I, "limit": 7.0}}
+    mem = {"type": "mlstm", "mixer": {"heads": D // 256, "dim": 128, "vdim": 256, "gate_cap": 15.0}, "mlp": None}
+    return BesulixConfig.from_dict({"architecture": "Besulix", "vocab": g["vocab_size"], "width": D, "norm": {"eps": 1e-6},
+                                    "logit_softcap": 30.0, "layers": [par if i % 2 == 0 else mem for i in range(n)]})
 
 
 def gemma_config(which, layers=0):
@@ -411,21 +430,156 @@ def time_lutovik_kernels(engine, cfg, batch, context, prefill_tokens):
     return out
 
 
+def time_besulix_kernels(engine, cfg, batch, context, prefill_tokens):
+    """Microseconds of Besulix's kernels at a decode step of `batch` sequences over `context` cached tokens and at a
+    prefill of `prefill_tokens`, each called once per layer on that layer's own weights, replayed from a HIP graph.
+    Products are priced by their weights' bytes (decode) or their flops against the bf16 matrix peak (prefill), the two
+    scans by their states' bytes (decode) or their multiply-adds against the float32 vector peak (prefill), the attention
+    by the cached rows it reads (decode) or its flops (prefill)."""
+    import torch
+    from .engine.batch import StepContext
+    model, ops, dev = engine.model, engine.model.rt.ops, engine.model.rt.device
+    bf, f32 = torch.bfloat16, torch.float32
+    blocks = [l.block for l in model.layers]
+    par = [b for b in blocks if hasattr(b.mixer, "sides")]
+    mem = [b for b in blocks if hasattr(b.mixer, "w_gates")]
+    dense = [b for b in blocks if b.feed_forward is not None]
+    D = cfg.hidden_size
+    out = {}
+    timed = _timer(dev, out)
+    cache = engine.cache
+    entry = lambda group: next(i for i, l in enumerate(model.layers) if l.block is group[0])
+    elems = lambda w: float(w.numel())
+    for rows, tag in ((batch, f"decode_b{batch}"), (prefill_tokens, f"prefill_{prefill_tokens}")):
+        decode = rows == batch
+        slots = [cache.acquire() for _ in range(batch if decode else 1)]
+        try:
+            for s in slots:
+                cache.grow(s, context if decode else rows)
+            counts = [1] * batch if decode else [rows]
+            starts = [context - 1] * batch if decode else [0]
+            ctx = StepContext(model.rt, cache, slots, counts, starts, [])
+            x = torch.randn((rows, D), device=dev).to(bf)
+            one = lambda f, **kw: timed(f"{tag}.{kw.pop('name')}", f, **kw)
+            prod = (lambda name, calls, w, m=rows: one(calls, name=name, bytes_each=2.0 * elems(w)) if decode
+                    else one(calls, name=name, flops_each=2.0 * m * elems(w)))
+            if par:
+                e = entry(par)
+                ctx.entry = ctx.cache_owner = e
+                left, right = par[0].mixer.sides
+                H, KV, row = left.num_heads, left.num_kv_heads, left.row
+                site = cache.site(e)
+                table = ctx.page_table(site.group_index)
+                kp, vp, cap = site.tensor("k"), site.tensor("v"), site.rows_cap or 0
+                prod("left_qkv_bias", [(lambda b=b: ops.linear(x, b.mixer.sides[0].w_qkv, bf, bias=b.mixer.sides[0].b_qkv)) for b in par], left.w_qkv)
+                qkv = torch.randn((rows, (H + 2 * KV) * row), device=dev).to(bf)
+                q, k, v = qkv[:, :H * row], qkv[:, H * row:(H + KV) * row], qkv[:, (H + KV) * row:]
+                one([lambda: left._turn(ctx, v, KV, left.value_freq)] * 16, name="turn_values", bytes_each=rows * KV * row * 4.0)
+                one([lambda: ops.rope_kv_write(q, k, v, H, KV, row, left.inv_freq, left.position.rotary_dim, ctx.row_seq, ctx.row_pos,
+                                               ctx.new_len, table, kp, vp, cap)] * 16, name="rope_kv_write", bytes_each=rows * (H + 3 * KV) * row * 4.0)
+                more = dict(chunk=left.chunk, head_scale=left.temperature, sink=left.sink)
+                seen = min(context, (context - 1) % left.chunk + 1) if left.chunk else context
+                if decode:
+                    one([lambda: ops.attention_decode(q, H, KV, row, ctx.new_len, table, kp, vp, cap, left.query_scale, 0.0, 0, bf,
+                                                  max_keys=ctx.max_rows_visible(site), **more)] * 8, name=f"attention_{seen}_of_{context}_keys",
+                        bytes_each=2.0 * batch * seen * 2 * KV * row)
+                else:
+                    C = left.chunk or rows
+                    full, rest = divmod(rows, C)
+                    pairs = full * C * (C + 1) / 2.0 + rest * (rest + 1) / 2.0
+                    one([lambda: ops.attention_prefill(q, k, v, H, KV, row, ctx.cu_rows, rows, left.query_scale, 0.0, 0, bf, row_seq=ctx.row_seq,
+                                                   row_pos=ctx.row_pos, wide_weights=left.precise_weights, **more)] * 4, name=f"attention_chunks_of_{C}", flops_each=4.0 * pairs * H * row)
+                heads_out = torch.randn((rows, H * row), device=dev).to(bf)
+                one([lambda: left._turn(ctx, heads_out, H, left.value_back)] * 16, name="turn_back", bytes_each=rows * H * row * 4.0)
+                prod("left_o", [(lambda b=b: ops.linear(heads_out, b.mixer.sides[0].w_o, f32)) for b in par], left.w_o)
+                # ---- the time-mixing side
+                nh, d, inner = right.num_heads, right.head_dim, right.inner
+                shift, memory = cache.entry_state(e, "mixer.right.shift"), cache.entry_state(e, "mixer.right.memory")
+                one([lambda: ops.shift_mix(x, right.mu, shift, ctx.slot_ids, ctx.cu_rows, ctx.row_seq, one_row_each=decode)] * 16,
+                    name="shift_mix", bytes_each=rows * D * 12.0)
+                for s in ("r", "g"):
+                    prod(f"right_{s}", [(lambda b=b, s=s: ops.linear(x, b.mixer.sides[1].w[s], bf)) for b in par], right.w[s])
+
+                def decay_rates(b):
+                    low = ops.unary_(ops.linear(x, b.mixer.sides[1].w["w1"], bf), "tanh")
+                    return ops.linear(low, b.mixer.sides[1].w["w2"], f32)
+                one([(lambda b=b: decay_rates(b)) for b in par], name="decay_w1_tanh_w2",
+                    bytes_each=2.0 * (elems(right.w["w1"]) + elems(right.w["w2"])) + rows * (D * 2.0 + inner * 4.0))
+                r_, k_, v_ = ((torch.randn((rows, inner), device=dev) * 0.3).to(bf) for _ in range(3))
+                rate = torch.randn((rows, inner), device=dev)
+                scan = lambda: ops.time_mix_scan(r_, k_, v_, rate, right.w0, right.bonus, memory, ctx.slot_ids, ctx.cu_rows,
+                                                 1 if decode else rows, nh, d)
+                if decode:
+                    one([scan] * 8, name="time_mix_scan", bytes_each=batch * nh * d * d * 8.0)
+                else:                                    # every row: the state's update and its product with r, 4 d d flop a head
+                    one([scan] * 4, name="time_mix_scan", flops_each=4.0 * rows * nh * d * d, peak=PEAK_FLOPS["float32"])
+                y = torch.randn((rows, inner), device=dev)
+                one([lambda: ops.head_norm_gate(y, right.norm_gain, r_, 1e-6, nh, "silu", bf)] * 16, name="head_norm_gate",
+                    bytes_each=rows * inner * 8.0)
+                yn = torch.randn((rows, inner), device=dev).to(bf)
+                prod("right_o", [(lambda b=b: ops.linear(yn, b.mixer.sides[1].w["o"], f32)) for b in par], right.w["o"])
+                oa, ob = torch.randn((rows, D), device=dev), torch.randn((rows, D), device=dev)
+                one([lambda: ops.weighted_sum(oa, 0.8, ob, 0.9)] * 16, name="weighted_sum", bytes_each=rows * D * 12.0)
+            if mem:
+                e = entry(mem)
+                ctx.entry = ctx.cache_owner = e
+                mm = mem[0].mixer
+                nh, dk, dv = mm.num_heads, mm.key_dim, mm.value_dim
+                prod("memory_in", [(lambda b=b: ops.linear(x, b.mixer.w_in, bf)) for b in mem], mm.w_in)
+                one([(lambda b=b: ops.linear(x, b.mixer.w_gates, f32, bias=b.mixer.b_gates)) for b in mem], name="memory_gates",
+                    bytes_each=2.0 * elems(mm.w_gates) + rows * D * 2.0)
+                u = (torch.randn((rows, mm.w_in.shape[0]), device=dev) * 0.3).to(bf)
+                gates = torch.randn((rows, 2 * nh), device=dev)
+                S, nrm, mx = (cache.entry_state(e, "mixer." + s) for s in ("memory", "normalizer", "maximum"))
+                qk, vv = nh * dk, nh * dv
+                scan = lambda: ops.matrix_memory_scan(u[:, :qk], u[:, qk:2 * qk], u[:, 2 * qk:2 * qk + vv], gates, mm.gate_cap, dk ** -0.5,
+                                                      S, nrm, mx, ctx.slot_ids, ctx.cu_rows, 1 if decode else rows, nh, dk, dv)
+                if decode:
+                    one([scan] * 8, name="matrix_memory_scan", bytes_each=batch * nh * dk * dv * 8.0)
+                else:
+                    one([scan] * 4, name="matrix_memory_scan", flops_each=4.0 * rows * nh * dk * dv, peak=PEAK_FLOPS["float32"])
+                y = torch.randn((rows, vv), device=dev)
+                one([lambda: ops.head_norm_gate(y, mm.norm_gain, u[:, 2 * qk + vv:2 * qk + 2 * vv], 1e-6, nh, "sigmoid", bf)] * 16,
+                    name="memory_head_norm_gate", bytes_each=rows * vv * 8.0)
+                yn = torch.randn((rows, vv), device=dev).to(bf)
+                prod("memory_o", [(lambda b=b: ops.linear(yn, b.mixer.w_o, bf, defer=True)) for b in mem], mm.w_o)
+            if dense:
+                ff = dense[0].feed_forward
+                prod("gate_up_clamped", [(lambda b=b: ops.gated_linear(x, b.feed_forward.w_gate_up, ff.intermediate_size, "quick_gelu", bf,
+                                                                       limit=ff.limit, up_shift=ff.up_shift)) for b in dense],
+                     ff.w_gate_up[:2 * ff.intermediate_size])
+                xi = torch.randn((rows, ff.intermediate_size), device=dev).to(bf)
+                prod("down", [(lambda b=b: ops.linear(xi, b.feed_forward.w_down, bf, defer=True)) for b in dense], ff.w_down)
+            stream = torch.randn((rows, D), device=dev)
+            rows_b = torch.randn((rows, D), device=dev).to(bf)
+            g = torch.ones(D, device=dev)
+            one([lambda: ops.add_rms_norm(stream, rows_b, None, 0.0, g, 1e-6, bf)] * 16, name="add_rms_norm",
+                bytes_each=rows * D * (4 + 4 + 2 + 2) + 4.0 * D)
+        finally:
+            for s in slots:
+                cache.release(s)
+    return out
+
+
 def main(args):
     import torch
     which = args.sizes
     steps, warmup = args.steps, max(2, args.warmup)
     prompt, batch = args.prompt, args.batch
     design = args.compare
-    build, time_design = {"golepel": (golepel_config, time_golepel_kernels), "lutovik": (lutovik_config, time_lutovik_kernels)}[design]
-    line = {"metric": f"{design.capitalize()} next to Gemma-2 at {which} layer sizes: prefill and decode tok/s", "unit": "tok/s", "n_gpus": 1,
+    build, time_design = {"golepel": (golepel_config, time_golepel_kernels), "lutovik": (lutovik_config, time_lutovik_kernels),
+                          "besulix": (besulix_config, time_besulix_kernels)}[design]
+    # the design it stands next to: the closest of the others
+    other, build_other, time_other, title = {"besulix": ("lutovik", lutovik_config, time_lutovik_kernels, "Lutovik")}.get(
+        design, ("gemma2", gemma_config, time_kernels, "Gemma-2"))
+    line = {"metric": f"{design.capitalize()} next to {title} at {which} layer sizes: prefill and decode tok/s", "unit": "tok/s", "n_gpus": 1,
             "steps": steps, "warmup": warmup, "dtype": "bf16", "data": "synthetic: seeded random weights N(0, 0.02) and uniform-random token ids",
             "sizes": which, "designs": {}, "kernels": {}}
     most = max(PREFILL_TOKENS, batch * (prompt + steps + warmup + 128)) + 1024
-    for name, cfg in ((design, build(which, args.layers)), ("gemma2", gemma_config(which, args.layers))):
+    for name, cfg in ((design, build(which, args.layers)), (other, build_other(which, args.layers))):
         run = Run(cfg, max(batch, 8), most, name)
         pre = run.prefill()
-        d = {"layers": len(cfg.layers) if name == design else cfg.num_hidden_layers, "weights_GB": round(run.weight_bytes / 1e9, 2),
+        d = {"layers": len(cfg.layers) if hasattr(cfg, "layers") else cfg.num_hidden_layers, "weights_GB": round(run.weight_bytes / 1e9, 2),
              f"prefill_{PREFILL_TOKENS}_tok_s": round(PREFILL_TOKENS / pre, 1), f"prefill_{PREFILL_TOKENS}_ms": round(pre * 1e3, 2)}
         for b in (batch, 1):
             dt = run.decode([prompt] * b, steps, warmup)
@@ -435,14 +589,14 @@ def main(args):
         if name == design:
             k = time_design(run.engine, cfg, batch, prompt + 40, PREFILL_TOKENS)
         else:
-            k = time_kernels(run.engine, cfg, batch, prompt + 40, PREFILL_TOKENS)
+            k = time_other(run.engine, cfg, batch, prompt + 40, PREFILL_TOKENS)
         for kn, row in k.items():
             print(f"[compare] {name} kernel {kn}: {row}", file=sys.stderr, flush=True)
         line["designs"][name] = d
         line["kernels"][name] = k
         run.close()
-    g, m = line["designs"][design], line["designs"]["gemma2"]
+    g, m = line["designs"][design], line["designs"][other]
     line["value"] = g[f"decode_b{batch}_tok_s"]
-    line["ratio_to_gemma2"] = {k: round(g[k] / m[k], 3) for k in g if k.endswith("tok_s")}
+    line[f"ratio_to_{other}"] = {k: round(g[k] / m[k], 3) for k in g if k.endswith("tok_s")}
     print(json.dumps(line), flush=True)
     return 0
