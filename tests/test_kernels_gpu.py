@@ -105,7 +105,7 @@ def test_rows_wider_than_the_fused_kernel_takes_are_added_first(ops):
     x, w = randn(8, 64, dtype=torch.bfloat16, seed=74), randn(128, 64, dtype=torch.bfloat16, seed=75)
     y = torch.empty(8, 128, dtype=torch.float32, device=DEV)
     ws = torch.empty(1 << 20, dtype=torch.uint8, device=DEV)
-    rc = ops.lib.tp_linear(x.data_ptr(), w.data_ptr(), y.data_ptr(), 1, 0, 8, 128, 64, 1, 30.0, 0, 0, ws.data_ptr(), 1 << 20, 1, 0, None)
+    rc = ops.lib.tp_linear(x.data_ptr(), w.data_ptr(), y.data_ptr(), 1, 0, 8, 128, 64, 1, 30.0, 0, 0, 0.0, 0.0, ws.data_ptr(), 1 << 20, 1, 0, None)
     assert rc != 0 and b"epilogue" in ops.lib.tp_last_error()
 
 
@@ -493,6 +493,74 @@ def test_attention_decode(ops, plain, dt, H, KV, hd, lens, page, window, rows_ca
     finally:
         ops.force_plain_attention = False
     assert rel_l2(got, ref) < (3e-6 if dt == "f32" else 8e-3)
+
+
+CHUNK_CASES = [
+    # H, KV, hd, lens, page, chunk, window, rows_cap, cap
+    (4, 2, 16, (5, 41, 17), 16, 20, 0, 0, 0.0),             # chunks that end inside a tile of keys
+    (6, 3, 64, (130, 64, 65), 64, 64, 0, 64, 0.0),          # a ring of one chunk
+    (8, 2, 128, (300, 99), 16, 100, 30, 0, 25.0),           # a window inside the chunk, capped scores
+    (2, 2, 48, (70,), 16, 1, 0, 16, 0.0),                   # a chunk of one position: the query's own key and the sink
+    (3, 1, 80, (33, 200), 16, 1000, 0, 0, 0.0),             # a chunk longer than every sequence
+    (16, 4, 256, (257, 31), 64, 96, 0, 0, 0.0),
+]
+
+
+_chunk_refs = {}
+
+
+def chunk_case(dt, case):
+    """The inputs of a case and what the slow functions make of them, computed once for all kernels."""
+    if (dt, case) not in _chunk_refs:
+        H, KV, hd, lens, page, chunk, window, rows_cap, cap = case
+        n_pages = 32
+        c = build_cache_case(DT[dt], H, KV, hd, lens, page, rows_cap, n_pages, 50)
+        scale = 1.0 / math.sqrt(hd * 0.6)
+        temp = (0.5 + torch.rand(H, generator=torch.Generator().manual_seed(5))).float()
+        sink = randn(H, seed=6).cpu().float() * 2.0
+        more = dict(chunk=chunk, head_scale=temp, sink=sink)
+        ref = ref_ops.attention_prefill(c["q"].cpu(), c["k"].cpu(), c["v"].cpu(), H, KV, hd, c["cu"], max(lens), scale,
+                                        cap, window, torch.float32, **more)
+        pools = [torch.full((n_pages, KV, page, hd), 7.0, dtype=DT[dt]) for _ in range(2)]
+        ref_ops.rope_kv_write(c["q"].cpu().clone(), c["k"].cpu().clone(), c["v"].cpu(), H, KV, hd, None, 0, c["row_seq"],
+                              c["row_pos"], c["new_len"], c["table"], pools[0], pools[1], rows_cap)
+        qlast = torch.stack([c["q"].cpu()[int(c["cu"][i + 1]) - 1] for i in range(len(lens))]).contiguous()
+        ref_one = ref_ops.attention_decode(qlast, H, KV, hd, c["new_len"], c["table"], pools[0], pools[1], rows_cap, scale,
+                                           cap, window, torch.float32, **more)
+        bare = ref_ops.attention_decode(qlast, H, KV, hd, c["new_len"], c["table"], pools[0], pools[1], rows_cap, scale,
+                                        cap, window, torch.float32, chunk=chunk, head_scale=temp)
+        assert rel_l2(bare, ref_one) > 0.05                 # the sink is no small matter in these cases
+        _chunk_refs[(dt, case)] = (c, scale, temp, sink, ref, pools, qlast, ref_one)
+    return _chunk_refs[(dt, case)]
+
+
+@pytest.mark.parametrize("kernel", ["plain", 0, 1, 2, 3])
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("case", CHUNK_CASES)
+def test_attention_in_chunks_with_temperatures_and_sinks(ops, kernel, dt, case):
+    """Keys of the query's own chunk only, a factor per head on the scores, a score without key that joins the sum: in
+    the plain kernels and the matrix-core kernels, many queries and one, the keys of one query in slices too."""
+    plain = kernel == "plain"
+    if dt == "f32" and not plain:
+        pytest.skip("float32 runs on the plain kernel only")
+    H, KV, hd, lens, page, chunk, window, rows_cap, cap = case
+    c, scale, temp, sink, ref, pools, qlast, ref_one = chunk_case(dt, case)
+    dev = dict(chunk=chunk, head_scale=temp.to(DEV), sink=sink.to(DEV))
+    tol = 3e-6 if dt == "f32" else 8e-3
+    ops.force_plain_attention = plain
+    try:
+        got = ops.attention_prefill(c["q"], c["k"], c["v"], H, KV, hd, c["cu"].to(DEV), max(lens), scale, cap, window,
+                                    DT[dt], row_seq=c["row_seq"].to(DEV), row_pos=c["row_pos"].to(DEV),
+                                    shape=0 if plain else kernel, **dev)
+        assert rel_l2(got, ref) < tol
+        if kernel in ("plain", 0):
+            for splits in (None,) if plain else (None, 1, 2, 5):
+                one = ops.attention_decode(qlast.to(DEV), H, KV, hd, c["new_len"].to(DEV), c["table"].to(DEV),
+                                           pools[0].to(DEV), pools[1].to(DEV), rows_cap, scale, cap, window, DT[dt],
+                                           max_keys=max(lens), splits=splits, **dev)
+                assert rel_l2(one, ref_one) < tol, splits
+    finally:
+        ops.force_plain_attention = False
 
 
 @pytest.mark.parametrize("splits", [None, 1, 3])

@@ -73,6 +73,9 @@ struct DecodeArgs {
     // kv heads the pools really have (0: KV).  Fewer than KV: the grid's kv heads are groups of query heads that share
     // pool head `kvh % pool_kv` (a cache with one row per token for all heads is read by every group)
     int pool_kv;
+    // chunk C > 0: the query sees keys from floor(p / C) C on only.  head_scale, sink ([H] or null): a factor on every
+    // head's scores; a score without key or value that joins every head's softmax sum once
+    int chunk; const float* head_scale; const float* sink;
 };
 
 namespace {
@@ -98,7 +101,8 @@ attn_decode_k(DecodeArgs a) {
     const int kvh = blockIdx.x, seq = blockIdx.y, split = blockIdx.z;
     const int G = a.H / a.KV;
     const int p = a.new_len[seq] - 1;
-    const int lo = a.window > 0 ? max(0, p - a.window + 1) : 0;
+    int lo = a.window > 0 ? max(0, p - a.window + 1) : 0;
+    if (a.chunk > 0) lo = max(lo, p / a.chunk * a.chunk);
     const int lo_al = lo & ~15;
     int chunk = (p + 1 - lo_al + a.nsplit - 1) / a.nsplit;
     chunk = (chunk + ROUND - 1) / ROUND * ROUND;
@@ -260,7 +264,8 @@ attn_decode_k(DecodeArgs a) {
 #pragma unroll
         for (int e = 0; e < 8; e++) acc[qi][e] = 0.f;
     float m_run = -INFINITY, l_run = 0.f;            // of query head c, over this wave's keys so far
-    const float soc = a.cap > 0.f ? a.scale / a.cap : 0.f;
+    const float scale_c = a.head_scale && c < G ? a.scale * a.head_scale[kvh * G + c] : a.scale;     // lane (c, g): query head c of the group
+    const float soc = a.cap > 0.f ? scale_c / a.cap : 0.f;
 
     for (int tb = tb0; tb < t_end; tb += ROUND) {
         if (tb != tb0 || late) load_round(tb, kf, vf);
@@ -273,7 +278,7 @@ attn_decode_k(DecodeArgs a) {
         for (int i = 0; i < 4; i++) {
             const int t = tb + g * 4 + i;
             const bool ok = t >= lo && t < t_end;
-            s[i] = ok ? score_of(s[i], a.scale, a.cap, soc) : -INFINITY;
+            s[i] = ok ? score_of(s[i], scale_c, a.cap, soc) : -INFINITY;
             mx = fmaxf(mx, s[i]);
         }
         mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
@@ -348,6 +353,7 @@ attn_decode_k(DecodeArgs a) {
             }
             const int head = kvh * G + qi;
             if (a.nsplit == 1) {
+                if (a.sink) den += __expf(a.sink[head] - mx);                 // (the slice holds the query's own key: mx is finite)
                 a.out[((size_t)seq * a.H + head) * HD + tid] = f32_to_bf16(num / den);
             } else {
                 const size_t at = ((size_t)seq * a.H + head) * a.nsplit + split;
@@ -364,7 +370,7 @@ attn_decode_k(DecodeArgs a) {
 // unwritten: its weight is zero and the value is replaced by zero).
 __global__ void __launch_bounds__(256)
 attn_decode_combine_k(const float* __restrict__ ws_o, const float* __restrict__ ws_ml, int nsplit,
-                      bf16_t* __restrict__ out) {
+                      bf16_t* __restrict__ out, const float* __restrict__ sink, int H) {
     __shared__ float w_lds[128];
     const size_t at = (size_t)blockIdx.x * nsplit;               // blockIdx.x = sequence * heads + head
     const int tid = threadIdx.x;
@@ -391,6 +397,7 @@ attn_decode_combine_k(const float* __restrict__ ws_o, const float* __restrict__ 
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         float den = 0.f;
         for (int s = 0; s < nsplit; s++) den += w_lds[s];
+        if (sink) den += __expf(sink[blockIdx.x % H] - mx);       // (some slice holds the query's own key: mx is finite)
         __builtin_amdgcn_wave_barrier();
         w_lds[tid] = w0 / den;
         w_lds[tid + 64] = w1 / den;
@@ -429,7 +436,9 @@ static int decode_launch(DecodeArgs a, int n_seq, void* workspace, hipStream_t s
     TP_REQUIRE(a.pool_kv > 0 && a.KV % a.pool_kv == 0 && (a.pool_kv == a.KV || !a.qkv),
                "attention decode: %d groups of heads cannot share %d kv heads of the cache", a.KV, a.pool_kv);
     TP_REQUIRE(a.page >= 16 && (a.page & (a.page - 1)) == 0 && a.table_w > 0, "attention decode (matrix-core kernel): page size %d must be a power of two, at least 16", a.page);
-    TP_REQUIRE(a.rows_cap == 0 || a.window <= a.rows_cap, "attention decode: a window of %d keys does not fit a ring of %d rows", a.window, a.rows_cap);
+    TP_REQUIRE(a.chunk >= 0, "attention decode: chunks of %d positions", a.chunk);
+    const int reach = a.window > 0 && a.chunk > 0 ? (a.window < a.chunk ? a.window : a.chunk) : (a.window > 0 ? a.window : a.chunk);
+    TP_REQUIRE(a.rows_cap == 0 || (reach > 0 && reach <= a.rows_cap), "attention decode: a reach of %d keys (window %d, chunk %d) does not fit a ring of %d rows", reach, a.window, a.chunk, a.rows_cap);
     TP_REQUIRE(a.rows_cap >= 0 && a.rows_cap % a.page == 0, "attention decode: ring of %d rows is no multiple of the page size %d", a.rows_cap, a.page);
     TP_REQUIRE(a.nsplit >= 1 && a.nsplit <= 128 && (a.nsplit == 1 || workspace), "attention decode: %d slices (at most 128) need a workspace", a.nsplit);
     TP_REQUIRE(a.KV <= 65535 && n_seq <= 65535, "attention decode: grid too large");
@@ -445,7 +454,7 @@ static int decode_launch(DecodeArgs a, int n_seq, void* workspace, hipStream_t s
     else attn_decode_k<16><<<grid, DTH, 0, s>>>(a);
     if (int rc = tp_check_launch("attention decode")) return rc;
     if (a.nsplit > 1) {
-        attn_decode_combine_k<<<n_seq * a.H, HD < 64 ? 64 : HD, 0, s>>>(a.ws_o, a.ws_ml, a.nsplit, a.out);
+        attn_decode_combine_k<<<n_seq * a.H, HD < 64 ? 64 : HD, 0, s>>>(a.ws_o, a.ws_ml, a.nsplit, a.out, a.sink, a.H);
         return tp_check_launch("attention decode (combine)");
     }
     return 0;
@@ -453,12 +462,12 @@ static int decode_launch(DecodeArgs a, int n_seq, void* workspace, hipStream_t s
 
 extern "C" int tp_attn_decode(const void* q, long q_stride, int n_seq, int H, int KV, const int* new_len,
                               const int* table, int table_w, const void* k_pool, const void* v_pool, int page,
-                              int rows_cap, float scale, float cap, int window, void* out, void* workspace,
-                              int nsplit, void* stream) {
+                              int rows_cap, float scale, float cap, int window, int chunk, const float* head_scale,
+                              const float* sink, void* out, void* workspace, int nsplit, void* stream) {
     TP_REQUIRE(q_stride % 8 == 0 && (uintptr_t)q % 16 == 0, "attention decode: query rows must be 16-byte aligned");
     DecodeArgs a{(const bf16_t*)q, q_stride, H, KV, new_len, table, table_w, (bf16_t*)k_pool, (bf16_t*)v_pool,
                  page, rows_cap, scale, cap, window, (bf16_t*)out, nullptr, nullptr, nsplit,
-                 nullptr, 0, 1, 0, 0, nullptr, 0, 0};
+                 nullptr, 0, 1, 0, 0, nullptr, 0, 0, 0, chunk, head_scale, sink};
     return decode_launch(a, n_seq, workspace, (hipStream_t)stream);
 }
 

@@ -52,6 +52,9 @@ struct PrefillArgs {
     int H, KV, ghb_shift, pt_shift;           // heads of a kv head a block takes: 1 << ghb_shift; its position tiles: 1 << pt_shift
     int n_streams, pos_blocks;                // (sequence, kv head, head group) triples; blocks of positions per stream
     float scale, cap; int window;
+    int chunk;                                // C > 0: the query at p sees keys from floor(p / C) C on only
+    const float* head_scale;                  // [H] or null: a factor on every head's scores
+    const float* sink;                        // [H] or null: a score without key or value that joins every softmax's sum once
     bf16_t* out;
 };
 
@@ -138,6 +141,7 @@ attn_prefill_k(PrefillArgs a) {
 
     // ---- the keys the block walks: tiles of 32 positions, aligned to multiples of 32 ---------------------------
     int k_lo = a.window > 0 ? max(0, start + q0 - a.window + 1) : 0;
+    if (a.chunk > 0) k_lo = max(k_lo, (start + q0) / a.chunk * a.chunk);     // the block's first query has the earliest chunk
     k_lo &= ~31;
     const int k_hi = min(L, start + q0 + PB);
     const int n_rounds = (k_hi - k_lo + 32 * KG - 1) / (32 * KG);
@@ -231,8 +235,13 @@ attn_prefill_k(PrefillArgs a) {
 #pragma unroll
         for (int e = 0; e < 16; e++) o[dt][e] = 0.f;
     float m_ref = -INFINITY, l_i = 0.f;                            // in units of log 2; l_i: this lane's 16 keys of every tile
-    const float tanh_in = a.cap > 0.f ? 2.f * LOG2E * a.scale / a.cap : 0.f, cap2 = a.cap * LOG2E, scale2 = a.scale * LOG2E;
-    const unsigned win = a.window > 0 ? (unsigned)a.window : 0x7fffffffu;
+    const float scale_h = a.head_scale ? a.scale * a.head_scale[h] : a.scale;
+    const float tanh_in = a.cap > 0.f ? 2.f * LOG2E * scale_h / a.cap : 0.f, cap2 = a.cap * LOG2E, scale2 = scale_h * LOG2E;
+    // keys a query sees behind it, itself included: the window, and what its chunk holds up to it
+    unsigned win = a.window > 0 ? (unsigned)a.window : 0x7fffffffu;
+    if (a.chunk > 0) win = min(win, (unsigned)(max(qpos, 0) % a.chunk) + 1u);
+    // the chunks' first positions for the wave's first and last query (wave-uniform)
+    const int chunk_first = a.chunk > 0 ? max(qw0, 0) / a.chunk * a.chunk : 0, chunk_last = a.chunk > 0 ? (max(qw0, 0) + 31) / a.chunk * a.chunk : 0;
 
     rows_of_round(0);
     issue_k();
@@ -257,7 +266,7 @@ attn_prefill_k(PrefillArgs a) {
     for (int r = 0; r < n_rounds; r++) {
         const int kt = k_lo + 32 * (r * KG + kg);
         // wave-uniform: some key of the tile is visible to some query of the wave
-        const bool visible = kt < k_hi && kt <= qw0 + 31 && qw0 < L && (a.window <= 0 || kt + 31 > qw0 - a.window);
+        const bool visible = kt < k_hi && kt <= qw0 + 31 && qw0 < L && (a.window <= 0 || kt + 31 > qw0 - a.window) && kt + 31 >= chunk_first;
         if (visible) {
             // two chains of accumulation where the registers allow it (at head size 256 they do not, and a second
             // chain measured no faster there: the SIMD's other wave fills in)
@@ -298,7 +307,7 @@ attn_prefill_k(PrefillArgs a) {
             issue_k();
         }
         if (visible) {
-            const bool whole = kt + 31 <= qw0 && (a.window <= 0 || qw0 + 31 - kt < a.window);
+            const bool whole = kt + 31 <= qw0 && (a.window <= 0 || qw0 + 31 - kt < a.window) && kt >= chunk_last;
             if (!whole) {
                 const int d0 = qpos - kt - 4 * hi;   // distance to key j: d0 - 8 (j / 4) - j % 4; visible: 0 <= distance < window
 #pragma unroll
@@ -404,7 +413,9 @@ attn_prefill_k(PrefillArgs a) {
         if (kg > 0) return;
     }
     if (!q_ok) return;
-    const float inv = 1.f / pair_sum(l_i);
+    float total = pair_sum(l_i);
+    if (a.sink) total += exp2_fast(a.sink[h] * LOG2E - m_ref);       // (a query sees its own key at least: m_ref is finite)
+    const float inv = 1.f / total;
     // lane: head elements dt * 32 + 8 (j / 4) + 4 hi + j % 4 of query `col`: four neighbours per store
     bf16_t* orow = a.out + ((size_t)(row0 + qpos - start) * a.H + h) * HD + 4 * hi;
 #pragma unroll
@@ -444,18 +455,21 @@ int prefill_launch(const PrefillArgs& a, int blocks, hipStream_t stream) {
 extern "C" int tp_attn_prefill(const void* q, long q_stride, const void* k, long k_stride, const void* v, long v_stride,
                                int M, int H, int KV, const int* cu_rows, int n_seq, int max_count,
                                const int* new_len, const int* table, int table_w, const void* k_pool, const void* v_pool,
-                               int page, int rows_cap, float scale, float cap, int window, void* out, int shape, void* stream) {
+                               int page, int rows_cap, float scale, float cap, int window, int chunk, const float* head_scale,
+                               const float* sink, void* out, int shape, void* stream) {
     TP_REQUIRE(M > 0 && H > 0 && KV > 0 && n_seq > 0 && max_count > 0, "attention prefill: empty shape");
     TP_REQUIRE(H % KV == 0, "attention: %d query heads are no multiple of %d kv heads", H, KV);
     TP_REQUIRE(q_stride % 8 == 0 && k_stride % 8 == 0 && v_stride % 8 == 0 && (uintptr_t)q % 16 == 0 &&
                (uintptr_t)k % 16 == 0 && (uintptr_t)v % 16 == 0, "attention prefill: rows must be 16-byte aligned");
     TP_REQUIRE(scale > 0.f, "attention prefill: the scale %g must be positive", scale);
+    TP_REQUIRE(chunk >= 0, "attention prefill: chunks of %d positions", chunk);
     const bool paged = new_len != nullptr;
     if (paged) {
         TP_REQUIRE(table && k_pool && v_pool && table_w > 0, "attention prefill: cached positions need the page table and the pools");
         TP_REQUIRE(page >= 16 && (page & (page - 1)) == 0, "attention prefill (matrix-core kernel): page size %d must be a power of two, at least 16", page);
         TP_REQUIRE(rows_cap >= 0 && rows_cap % page == 0, "attention prefill: ring of %d rows is no multiple of the page size %d", rows_cap, page);
-        TP_REQUIRE(rows_cap == 0 || (window > 0 && window <= rows_cap), "attention prefill: a window of %d keys does not fit a ring of %d rows", window, rows_cap);
+        const int reach = window > 0 && chunk > 0 ? (window < chunk ? window : chunk) : (window > 0 ? window : chunk);
+        TP_REQUIRE(rows_cap == 0 || (reach > 0 && reach <= rows_cap), "attention prefill: a reach of %d keys (window %d, chunk %d) does not fit a ring of %d rows", reach, window, chunk, rows_cap);
         TP_REQUIRE((uintptr_t)k_pool % 16 == 0 && (uintptr_t)v_pool % 16 == 0, "attention prefill: the pools must be 16-byte aligned");
     }
     const int G = H / KV;
@@ -467,6 +481,7 @@ extern "C" int tp_attn_prefill(const void* q, long q_stride, const void* k, long
     while (paged && (1 << ps) < page) ps++;
     a.page_shift = ps; a.page_mask = page - 1; a.rows_cap = paged ? rows_cap : 0;
     a.H = H; a.KV = KV; a.scale = scale; a.cap = cap; a.window = window; a.out = (bf16_t*)out;
+    a.chunk = chunk; a.head_scale = head_scale; a.sink = sink;
     static int cus = 0;
     if (!cus) {
         int dev = 0;

@@ -55,8 +55,8 @@ _CORE_SIGS = {
     "tp_probe_mfma": [_I, _I, _I, _P, _P, _P],
 }
 _ATTN_SIGS = {
-    "tp_attn_prefill": [_P, _L, _P, _L, _P, _L, _I, _I, _I, _P, _I, _I, _P, _P, _I, _P, _P, _I, _I, _F, _F, _I, _P, _I, _P],
-    "tp_attn_decode": [_P, _L, _I, _I, _I, _P, _P, _I, _P, _P, _I, _I, _F, _F, _I, _P, _P, _I, _P],
+    "tp_attn_prefill": [_P, _L, _P, _L, _P, _L, _I, _I, _I, _P, _I, _I, _P, _P, _I, _P, _P, _I, _I, _F, _F, _I, _I, _P, _P, _P, _I, _P],
+    "tp_attn_decode": [_P, _L, _I, _I, _I, _P, _P, _I, _P, _P, _I, _I, _F, _F, _I, _I, _P, _P, _P, _P, _I, _P],
     "tp_attn_decode_shared": [_P, _L, _I, _I, _I, _I, _P, _P, _I, _P, _P, _I, _I, _F, _F, _I, _P, _P, _I, _P],
     "tp_attn_decode_workspace_floats": [_I, _I, _I],
     "tp_attn_decode_fused": [_P, _I, _I, _L, _L, _P, _I, _I, _I, _I, _I, _P, _P, _I, _P, _P, _I, _I, _F, _F, _I, _P, _P, _I, _P],
@@ -770,10 +770,9 @@ class HipOps:
         wide_weights: the matrix-core kernel multiplies the values by softmax weights of 16 bits of mantissa (two bf16
         terms) instead of 8; the plain kernel's weights are float32 in any case.
         chunk C: a query at position p sees keys from floor(p / C) C on only.  head_scale, sink: float32 [H], a factor on
-        every head's scores and a score without key or value in every head's softmax.  With any of the three the step
-        runs on the plain kernel (the matrix-core kernels have none of them)."""
+        every head's scores and a score without key or value in every head's softmax."""
         self._dev(q, k, v, cu_rows, head_scale, sink)
-        plain_only = self._head_vectors("attention_prefill", H, chunk, head_scale, sink)
+        self._head_vectors("attention_prefill", H, chunk, head_scale, sink)
         m = q.shape[0]
         qs, ks, vs = self._rows(q, "attention q"), self._rows(k, "attention k"), self._rows(v, "attention v")
         if q.shape[1] != H * hd or k.shape != (m, KV * hd) or v.shape != (m, KV * hd):
@@ -790,12 +789,13 @@ class HipOps:
             page, table_w, rows_cap = k_pool.shape[2], table.shape[1], rows_cap or 0
         ptr = lambda t: t.data_ptr() if t is not None else None
         out = torch.empty((m, H * hd), dtype=out_dtype, device=self.device)
-        if not plain_only and self._fast_attention(q.dtype, H, KV, hd, decode=False) and (cached is None or (page >= 16 and page & (page - 1) == 0)):
+        if self._fast_attention(q.dtype, H, KV, hd, decode=False) and (cached is None or (page >= 16 and page & (page - 1) == 0)):
             lib = self.attn_lib(hd, wide=wide_weights)
             self._call(lib, "tp_attn_prefill", q.data_ptr(), qs, k.data_ptr(), ks, v.data_ptr(), vs,
                        m, H, KV, cu_rows.data_ptr(), n_seq, int(max_count), ptr(new_len), ptr(table), table_w,
                        ptr(k_pool), ptr(v_pool), page, rows_cap,
-                       float(scale), float(softcap), int(window), out.data_ptr(), int(shape), self._stream())
+                       float(scale), float(softcap), int(window), int(chunk), ptr(head_scale), ptr(sink), out.data_ptr(), int(shape),
+                       self._stream())
             return out
         if cached is not None and (row_seq is None or row_pos is None):
             raise KernelError("attention_prefill: cached positions need every row's sequence and position")
@@ -810,7 +810,7 @@ class HipOps:
         return out
 
     def _head_vectors(self, what, H, chunk, head_scale, sink):
-        """Checks what only the plain attention kernel takes; whether any of it is asked for."""
+        """Checks a chunk size and the vectors of one number per head; whether any of them is asked for."""
         if chunk < 0:
             raise KernelError(f"{what}: chunks of {chunk} positions")
         for t, name in ((head_scale, "head_scale"), (sink, "sink")):
@@ -844,7 +844,7 @@ class HipOps:
         otherwise form all their weighted sums.  The plain kernel takes any grouping as it is.
         chunk, head_scale, sink: as in `attention_prefill`."""
         self._dev(q, new_len, table, k_pool, v_pool, head_scale, sink)
-        plain_only = self._head_vectors("attention_decode", H, chunk, head_scale, sink)
+        per_head = self._head_vectors("attention_decode", H, chunk, head_scale, sink)
         n = q.shape[0]
         qs = self._rows(q, "attention q")
         if q.shape[1] != H * hd:
@@ -855,7 +855,7 @@ class HipOps:
         groups = int(head_groups) if head_groups else KV
         if groups % KV or H % groups:
             raise KernelError(f"attention_decode: {H} heads in {groups} groups on {KV} kv heads")
-        if not plain_only and self._fast_attention(q.dtype, H, groups, hd) and page >= 16 and page & (page - 1) == 0:
+        if self._fast_attention(q.dtype, H, groups, hd) and page >= 16 and page & (page - 1) == 0 and not (per_head and groups != KV):
             lib = self.attn_lib(hd)
             keys = int(max_keys) if max_keys else k_pool.shape[0] * k_pool.shape[2]
             nsplit = int(splits) if splits else self.decode_splits(n, groups, hd, keys)
@@ -869,7 +869,8 @@ class HipOps:
                 return out
             self._call(lib, "tp_attn_decode", q.data_ptr(), qs, n, H, KV, new_len.data_ptr(), table.data_ptr(),
                        table.shape[1], k_pool.data_ptr(), v_pool.data_ptr(), k_pool.shape[2], rows_cap, float(scale),
-                       float(softcap), int(window), out.data_ptr(), ws.data_ptr() if ws is not None else None, nsplit,
+                       float(softcap), int(window), int(chunk), head_scale.data_ptr() if head_scale is not None else None,
+                       sink.data_ptr() if sink is not None else None, out.data_ptr(), ws.data_ptr() if ws is not None else None, nsplit,
                        self._stream())
             return out
         self._call(self.lib, "tp_attn_simple_decode", q.data_ptr(), qs, _code(q.dtype), n, H, KV, hd, new_len.data_ptr(),

@@ -31,7 +31,7 @@ def build_spec(c: BesulixConfig) -> ModelSpec:
             left = ("attention", {"hidden_size": D, "num_heads": a.heads, "num_kv_heads": a.kv_heads, "head_dim": a.dim,
                                   "value_dim": a.vdim, "query_scale": a.scale, "position": position,
                                   "tensors": ("q", "k", "v", "o"), "bias_suffix": ".b", "chunk": a.chunk,
-                                  "head_temperature": "temp", "sink": "sink", "value_rotation": a.rot.base})
+                                  "head_temperature": "temp", "sink": "sink", "value_rotation": a.rot.base, "precise_weights": True})
             right = ("time_mix", {"hidden_size": D, "num_heads": r.heads, "head_dim": r.dim, "norm_eps": c.norm_eps})
             mixer = ("parallel", {"hidden_size": D, "left": left, "right": right, "combine": "weighted_sum",
                                   "weights": (m.left_scale, m.right_scale)})

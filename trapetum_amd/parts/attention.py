@@ -27,8 +27,10 @@ sequence's first position (the cache then keeps a ring of C positions); a temper
 scores; a sink per head, a learned score without key or value whose exponential joins the softmax's denominator once;
 and `value_rotation` theta: the value of position t is turned by t over all its elements like a key (pairs (d, d +
 value_dim / 2), frequencies theta^(-2d / value_dim)) before it is cached, and a head's output at position p is turned
-back by -p, so that the weighted sum is read in the query's frame.  With any of the last four the step runs on the
-plain kernel, which keeps scores and weights in float32.
+back by -p, so that the weighted sum is read in the query's frame.  Chunks, temperatures and sinks are arguments of
+every attention kernel (a chunk is a window whose start does not move with the query; the sink is added to the sum
+when a query's keys are done, in the kernel that normalises); the values' two rotations are launches of the rotation
+kernel.  A decode step of such a layer is not the one fused launch: its projections carry biases and its values turn.
 """
 from ..cache.store import TokenSpec
 from ..models.spec import TensorSpec
@@ -78,9 +80,8 @@ class Attention(Mixer):
         if value_rotation is not None:
             self.value_position = build_part("position", ("rope", {"rotary_dim": self.value_dim, "theta": value_rotation}))
         self.output_dtype = None         # a mixer that holds this one may ask for its last product in another dtype
-        # the kernels of the matrix cores know none of these: such an attention runs on the plain kernel
-        self.plain_only = bool(self.chunk or head_temperature or sink or value_rotation is not None)
-        if self.plain_only and (self.output_gate or not self.own_kv):
+        self.per_head = bool(self.chunk or head_temperature or sink)
+        if (self.per_head or value_rotation is not None) and (self.output_gate or not self.own_kv):
             raise ValueError("chunks, temperatures, sinks and rotated values go with an ungated attention on its own cache")
 
     @property
@@ -180,9 +181,8 @@ class Attention(Mixer):
         k_pool, v_pool = site.tensor("k"), site.tensor("v")         # [pages, kv_heads, page, row]
         rows_cap = site.rows_cap or 0
         bias = None if self.b_qkv is None else (self.b_qkv if owns_cache else self.b_qkv[:Q])
-        # what the plain kernel takes beyond the others: see the module's text
-        more = dict(chunk=self.chunk, head_scale=self.temperature, sink=self.sink) if self.plain_only else {}
-        if ctx.mode == "decode" and bias is None and not self.plain_only and ops.fuses_decode_step(ctx.dtype, H, KV, hd, k_pool):
+        more = dict(chunk=self.chunk, head_scale=self.temperature, sink=self.sink) if self.per_head else {}
+        if ctx.mode == "decode" and bias is None and not self.per_head and self.value_freq is None and ops.fuses_decode_step(ctx.dtype, H, KV, hd, k_pool):
             # one launch rotates, writes the cache and attends; the projections may stay in K slices until then
             qkv = ops.linear(x, w_in, ctx.dtype, defer=True)
             out = ops.attention_decode_step(qkv, H, KV, hd, self.inv_freq, self.position.rotary_dim, ctx.new_len,
