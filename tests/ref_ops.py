@@ -377,13 +377,15 @@ def unary_(x, name):
     return x
 
 
-def time_mix_scan(r, k, v, log_rate, w0, bonus, state, slot_ids, cu_rows, max_count, heads, dim):
+def time_mix_scan(r, k, v, log_rate, w0, bonus, state, slot_ids, cu_rows, max_count, heads, dim, chunk=None):
     """o = (S + diag(bonus) k v^T)^T r, then S <- diag(w) S + k v^T with w = exp(-exp(log_rate + w0)), row after row of
     every sequence from state[slot] [heads, dim, dim], which is left updated.  float32 [M, heads dim]."""
     m = r.shape[0]
-    rf, kf, vf = (t.float().reshape(m, heads, dim) for t in (r, k, v))
-    w = torch.exp(-torch.exp(log_rate.float() + w0)).reshape(m, heads, dim)
-    y = torch.empty((m, heads, dim), dtype=torch.float32, device=r.device)
+    wide = state.dtype                                   # float64 states: the whole recurrence in float64
+    rf, kf, vf = (t.to(wide).reshape(m, heads, dim) for t in (r, k, v))
+    w = torch.exp(-torch.exp(log_rate.to(wide) + w0.to(wide))).reshape(m, heads, dim)
+    bonus = bonus.to(wide)
+    y = torch.empty((m, heads, dim), dtype=wide, device=r.device)
     for i in range(len(cu_rows) - 1):
         slot = int(slot_ids[i])
         S = state[slot].clone()
@@ -392,18 +394,19 @@ def time_mix_scan(r, k, v, log_rate, w0, bonus, state, slot_ids, cu_rows, max_co
             y[t] = torch.einsum("hkv,hk->hv", S + bonus[:, :, None] * kv, rf[t])
             S = w[t][:, :, None] * S + kv
         state[slot] = S
-    return y.reshape(m, heads * dim)
+    return y.reshape(m, heads * dim).float()
 
 
-def matrix_memory_scan(q, k, v, gates, cap, q_scale, memory, normalizer, maximum, slot_ids, cu_rows, max_count, heads, dk, dv):
+def matrix_memory_scan(q, k, v, gates, cap, q_scale, memory, normalizer, maximum, slot_ids, cu_rows, max_count, heads, dk, dv, chunk=None):
     """gates float32 [M, 2 heads]: the input and forget gates' sums.  i = cap tanh(. / cap), f = logsigmoid(cap tanh(. / cap)),
     m' = max(f + m, i), S <- e^(f + m - m') S + e^(i - m') k v^T, n likewise with k, o = S^T q' / (max(|n . q'|, e^(-m')) + 1e-6)
     with q' = q q_scale; the states [slots, heads, dk, dv], [slots, heads, dk], [slots, heads] are left updated."""
     M = q.shape[0]
-    qf, kf, vf = q.float().reshape(M, heads, dk) * q_scale, k.float().reshape(M, heads, dk), v.float().reshape(M, heads, dv)
-    gi = cap * torch.tanh(gates[:, :heads].float() / cap)
-    gf = torch.nn.functional.logsigmoid(cap * torch.tanh(gates[:, heads:].float() / cap))
-    y = torch.empty((M, heads, dv), dtype=torch.float32, device=q.device)
+    wide = memory.dtype                                  # float64 states: the whole recurrence in float64
+    qf, kf, vf = q.to(wide).reshape(M, heads, dk) * q_scale, k.to(wide).reshape(M, heads, dk), v.to(wide).reshape(M, heads, dv)
+    gi = cap * torch.tanh(gates[:, :heads].to(wide) / cap)
+    gf = torch.nn.functional.logsigmoid(cap * torch.tanh(gates[:, heads:].to(wide) / cap))
+    y = torch.empty((M, heads, dv), dtype=wide, device=q.device)
     for s in range(len(cu_rows) - 1):
         slot = int(slot_ids[s])
         S, n, mx = memory[slot].clone(), normalizer[slot].clone(), maximum[slot].clone()
@@ -416,7 +419,7 @@ def matrix_memory_scan(q, k, v, gates, cap, q_scale, memory, normalizer, maximum
             den = torch.maximum((n * qf[t]).sum(-1).abs(), torch.exp(-mx)) + 1e-6
             y[t] = torch.einsum("hkv,hk->hv", S, qf[t]) / den[:, None]
         memory[slot], normalizer[slot], maximum[slot] = S, n, mx
-    return y.reshape(M, heads * dv)
+    return y.reshape(M, heads * dv).float()
 
 
 def head_norm_gate(y, gain, g, eps, heads, activation, out_dtype):

@@ -158,6 +158,40 @@ def test_time_mix_keeps_its_first_tokens(rt, cut):
     assert rel_l2(plain.time_mix(x2, W, "", sizes, EPS)[200:], want[200:]) > 0.3
 
 
+SCAN_LENS = (1, 7, 33, 64, 97, 130, 300)
+SCAN_SLOTS = (5, 0, 3, 9, 1, 7, 2)
+
+
+def scan_geometry(rt):
+    cu = torch.tensor([0] + list(torch.tensor(SCAN_LENS).cumsum(0)), dtype=torch.int32)
+    return cu, torch.tensor(SCAN_SLOTS, dtype=torch.int32), sum(SCAN_LENS)
+
+
+@pytest.mark.parametrize("chunk", [0, None, 4, 32, 50])
+@pytest.mark.parametrize("heads,dim", [(3, 20), (2, 64), (1, 130)])
+def test_time_mix_scan_in_chunks(rt, heads, dim, chunk):
+    """Sequences of unequal lengths from states that are not zero, in chunks of several sizes (a last chunk of one row, a
+    sequence shorter than a chunk, one exactly a chunk long): the outputs and the states left behind are those of the
+    rows taken one after the other.  The decays range from almost none to almost all."""
+    from . import ref_ops
+    cu, slots, M = scan_geometry(rt)
+    inner = heads * dim
+    r, k, v = (rnd(M, inner, seed=60 + i, scale=0.5) for i in range(3))
+    rate = rnd(M, inner, seed=63, scale=2.0) - 2.0
+    w0, bonus = rnd(inner, seed=64, scale=0.5), rnd(heads, dim, seed=65, scale=0.5)
+    state = rnd(10, heads, dim, dim, seed=66, scale=0.3)
+    rd, kd, vd = (acts(rt, t)[0] for t in (r, k, v))
+    want_state = state.double()
+    want = ref_ops.time_mix_scan(rd.cpu(), kd.cpu(), vd.cpu(), rate, w0, bonus, want_state, slots, cu, max(SCAN_LENS), heads, dim)
+    got_state = state.to(rt.device)
+    got = rt.ops.time_mix_scan(rd, kd, vd, rate.to(rt.device), w0.to(rt.device), bonus.to(rt.device), got_state, slots.to(rt.device),
+                               cu.to(rt.device), max(SCAN_LENS), heads, dim, chunk=chunk)
+    for i in range(len(SCAN_LENS)):
+        assert rel_l2(got[cu[i]:cu[i + 1]], want[cu[i]:cu[i + 1]]) < 5e-6, i
+        assert rel_l2(got_state[SCAN_SLOTS[i]], want_state[SCAN_SLOTS[i]].float()) < 5e-6, i
+    assert torch.equal(got_state[[4, 6, 8]].cpu(), state[[4, 6, 8]])          # slots of no sequence are left alone
+
+
 # ---- the matrix memory --------------------------------------------------------------------------------------------------------
 def matrix_memory_tensors(heads, dim, vdim, seed=0, i_bias=0.0, f_bias=1.0, gate_scale=0.3):
     return {"q": rnd(heads * dim, WIDTH, seed=seed + 1, scale=0.25), "k": rnd(heads * dim, WIDTH, seed=seed + 2, scale=0.25),
@@ -186,6 +220,35 @@ def test_matrix_memory_part(rt, heads, dim, vdim, cap, i_bias, gate_scale):
     for i in seqs:
         # bfloat16: the denominator max(|n . q|, e^(-m)) turns small now and then, and the rounding of q and k with it
         assert rel_l2(got[i][0], plain.matrix_memory(wide[i], W, "", sizes, EPS)) < PART_TOL[rt.dtype] * (3 if rt.dtype == torch.float32 else 6), i
+
+
+@pytest.mark.parametrize("chunk", [0, None, 4, 32, 50])
+@pytest.mark.parametrize("heads,dk,dv,i_bias", [(3, 20, 36, 0.0), (2, 64, 128, 6.0), (1, 130, 70, -6.0), (2, 32, 200, 0.0)])
+def test_matrix_memory_scan_in_chunks(rt, heads, dk, dv, i_bias, chunk):
+    """As for the time-mixing scan; the running maximum starts from states above and below what the chunks reach."""
+    from . import ref_ops
+    cu, slots, M = scan_geometry(rt)
+    q, k = rnd(M, heads * dk, seed=70, scale=0.5), rnd(M, heads * dk, seed=71, scale=0.5)
+    v = rnd(M, heads * dv, seed=72, scale=0.5)
+    gates = torch.cat([rnd(M, heads, seed=73, scale=3.0) + i_bias, rnd(M, heads, seed=74, scale=3.0) + 1.0], dim=1).contiguous()
+    S, n = rnd(10, heads, dk, dv, seed=75, scale=0.3), rnd(10, heads, dk, seed=76, scale=0.3)
+    mx = rnd(10, heads, seed=77, scale=4.0)
+    qd, kd, vd = (acts(rt, t)[0] for t in (q, k, v))
+    want_states = [S.double(), n.double(), mx.double()]
+    want = ref_ops.matrix_memory_scan(qd.cpu(), kd.cpu(), vd.cpu(), gates, 8.0, dk ** -0.5, *want_states, slots, cu, max(SCAN_LENS), heads, dk, dv)
+    got_states = [t.to(rt.device) for t in (S, n, mx)]
+    got = rt.ops.matrix_memory_scan(qd, kd, vd, gates.to(rt.device), 8.0, dk ** -0.5, *got_states, slots.to(rt.device), cu.to(rt.device),
+                                    max(SCAN_LENS), heads, dk, dv, chunk=chunk)
+    for i in range(len(SCAN_LENS)):
+        # (max(|n . q|, e^(-m)) is a small difference of large terms now and then: float32 against float64, in any cut)
+        assert rel_l2(got[cu[i]:cu[i + 1]], want[cu[i]:cu[i + 1]]) < 6e-5, i
+        # a state is kept in units of e^(its maximum): compare what the pair stands for
+        for g, w in zip(got_states[:2], want_states[:2]):
+            lift = lambda t, m: t[SCAN_SLOTS[i]].cpu().double() * torch.exp(m[SCAN_SLOTS[i]].cpu().double()).reshape(heads, *([1] * (t.dim() - 2)))
+            assert rel_l2(lift(g, got_states[2]), lift(w, want_states[2])) < 1e-5, i
+        assert torch.allclose(got_states[2][SCAN_SLOTS[i]].cpu(), want_states[2][SCAN_SLOTS[i]].float(), atol=1e-5, rtol=1e-6), i
+    for g, w in zip(got_states, (S, n, mx)):
+        assert torch.equal(g[[4, 6, 8]].cpu(), w[[4, 6, 8]])
 
 
 @pytest.mark.parametrize("cut", ["whole", "pieces", "one by one"])

@@ -529,7 +529,7 @@ def chunk_case(dt, case):
                                            cap, window, torch.float32, **more)
         bare = ref_ops.attention_decode(qlast, H, KV, hd, c["new_len"], c["table"], pools[0], pools[1], rows_cap, scale,
                                         cap, window, torch.float32, chunk=chunk, head_scale=temp)
-        assert rel_l2(bare, ref_one) > 0.05                 # the sink is no small matter in these cases
+        assert rel_l2(bare, ref_one) > 0.01                 # the sink is no small matter in these cases
         _chunk_refs[(dt, case)] = (c, scale, temp, sink, ref, pools, qlast, ref_one)
     return _chunk_refs[(dt, case)]
 

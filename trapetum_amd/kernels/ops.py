@@ -39,8 +39,10 @@ _CORE_SIGS = {
     "tp_unary_tanh": [_P, _I, _L, _P],
     "tp_weighted_sum": [_P, _F, _P, _F, _I, _P, _L, _P],
     "tp_head_norm_gate": [_P, _P, _P, _L, _I, _F, _P, _I, _I, _I, _I, _I, _P],
-    "tp_time_mix_scan": [_P, _L, _P, _L, _P, _L, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _P],
-    "tp_matrix_memory_scan": [_P, _L, _P, _L, _P, _L, _I, _P, _F, _F, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
+    "tp_time_mix_scan": [_P, _L, _P, _L, _P, _L, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _P],
+    "tp_matrix_memory_scan": [_P, _L, _P, _L, _P, _L, _I, _P, _F, _F, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _P],
+    "tp_time_mix_scan_workspace_floats": [_I, _I, _I, _I],
+    "tp_matrix_memory_scan_workspace_floats": [_I, _I, _I, _I, _I],
     "tp_linear_workspace_bytes": [_I, _I, _I, _I, _I, _I, _I, _I, _I],
     "tp_attn_simple_prefill": [_P, _L, _P, _L, _P, _L, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _F, _F, _I, _I, _P, _P, _P, _P],
     "tp_attn_simple_decode": [_P, _L, _I, _I, _I, _I, _I, _P, _P, _I, _P, _P, _I, _I, _F, _F, _I, _I, _P, _P, _P, _P],
@@ -533,11 +535,12 @@ class HipOps:
 
     MAX_SCAN_DIM = 256             # key rows a lane of a scan keeps of its column, and columns of a block
 
-    def time_mix_scan(self, r, k, v, log_rate, w0, bonus, state, slot_ids, cu_rows, max_count, heads, dim):
+    def time_mix_scan(self, r, k, v, log_rate, w0, bonus, state, slot_ids, cu_rows, max_count, heads, dim, chunk=None):
         """o = (S + diag(bonus) k v^T)^T r, then S <- diag(w) S + k v^T with w = exp(-exp(log_rate + w0)), row after row
         of every sequence from state[slot] (float32 [slots, heads, dim, dim]: key row, value column), which is left
         updated.  r, k, v [M, heads dim], possibly views of wider rows; log_rate float32 [M, heads dim]; w0 float32
-        [heads dim]; bonus float32 [heads, dim].  Returns float32 [M, heads dim]."""
+        [heads dim]; bonus float32 [heads, dim].  Returns float32 [M, heads dim].  chunk: rows of a chunk (0: whole
+        sequences; None: `scan_chunks` decides by max_count, which no sequence's rows may exceed)."""
         self._dev(r, k, v, log_rate, w0, bonus, state, slot_ids, cu_rows)
         m, inner = r.shape[0], heads * dim
         rs, ks, vs = self._rows(r, "time_mix_scan r"), self._rows(k, "time_mix_scan k"), self._rows(v, "time_mix_scan v")
@@ -554,17 +557,35 @@ class HipOps:
             raise KernelError(f"time_mix_scan: the state must be contiguous float32 [slots, {heads}, {dim}, {dim}]")
         n_seq = self._geometry("time_mix_scan", m, slot_ids, cu_rows)
         y = torch.empty((m, inner), dtype=torch.float32, device=self.device)
+        chunk, n_chunks = self.scan_chunks(max_count) if chunk is None else (int(chunk), -(-int(max_count) // int(chunk)) if chunk else 0)
+        ws = None
+        if chunk:
+            ws = torch.empty(self.lib.tp_time_mix_scan_workspace_floats(n_seq, n_chunks, heads, dim), dtype=torch.float32, device=self.device)
         self._call(self.lib, "tp_time_mix_scan", r.data_ptr(), rs, k.data_ptr(), ks, v.data_ptr(), vs, _code(r.dtype), log_rate.data_ptr(),
                    w0.data_ptr(), bonus.data_ptr(), state.data_ptr(), slot_ids.data_ptr(), cu_rows.data_ptr(), y.data_ptr(), n_seq, heads, dim,
-                   self._stream())
+                   chunk, n_chunks, ws.data_ptr() if ws is not None else None, self._stream())
         return y
 
-    def matrix_memory_scan(self, q, k, v, gates, cap, q_scale, memory, normalizer, maximum, slot_ids, cu_rows, max_count, heads, dk, dv):
+    SCAN_CHUNK_FROM = 96         # rows of the longest sequence from which a scan runs in chunks
+
+    def scan_chunks(self, max_count):
+        """(rows of a chunk, chunks that cover the longest sequence) for the two scans of a matrix state; (0, 0): every
+        sequence in one piece, row after row.  Chunks of 32 rows give a prompt of a few thousand tokens as many waves
+        as the chip has places for; longer ones take longer chunks, so that the states between them stay small."""
+        n = int(max_count)
+        if n < self.SCAN_CHUNK_FROM:
+            return 0, 0
+        chunk = 32 if n <= 8192 else 64 if n <= 32768 else 128
+        return chunk, -(-n // chunk)
+
+    def matrix_memory_scan(self, q, k, v, gates, cap, q_scale, memory, normalizer, maximum, slot_ids, cu_rows, max_count, heads, dk, dv,
+                           chunk=None):
         """gates float32 [M, 2 heads]: the input gates' sums, then the forget gates'.  i = cap tanh(. / cap),
         f = logsigmoid(cap tanh(. / cap)), m' = max(f + m, i), S <- e^(f + m - m') S + e^(i - m') k v^T, n likewise with k,
         o = S^T q' / (max(|n . q'|, e^(-m')) + 1e-6) with q' = q q_scale, row after row of every sequence from the states
         memory [slots, heads, dk, dv], normalizer [slots, heads, dk] and maximum [slots, heads] (float32), which are left
-        updated.  q, k [M, heads dk] and v [M, heads dv] may be views of wider rows.  Returns float32 [M, heads dv]."""
+        updated.  q, k [M, heads dk] and v [M, heads dv] may be views of wider rows.  Returns float32 [M, heads dv].
+        chunk: as in `time_mix_scan`."""
         self._dev(q, k, v, gates, memory, normalizer, maximum, slot_ids, cu_rows)
         m = q.shape[0]
         qs, ks, vs = self._rows(q, "matrix_memory_scan q"), self._rows(k, "matrix_memory_scan k"), self._rows(v, "matrix_memory_scan v")
@@ -583,9 +604,14 @@ class HipOps:
             raise KernelError("matrix_memory_scan: the gates' cap must be positive")
         n_seq = self._geometry("matrix_memory_scan", m, slot_ids, cu_rows)
         y = torch.empty((m, heads * dv), dtype=torch.float32, device=self.device)
+        chunk, n_chunks = self.scan_chunks(max_count) if chunk is None else (int(chunk), -(-int(max_count) // int(chunk)) if chunk else 0)
+        ws = None
+        if chunk:
+            ws = torch.empty(self.lib.tp_matrix_memory_scan_workspace_floats(n_seq, n_chunks, heads, dk, dv), dtype=torch.float32, device=self.device)
         self._call(self.lib, "tp_matrix_memory_scan", q.data_ptr(), qs, k.data_ptr(), ks, v.data_ptr(), vs, _code(q.dtype), gates.data_ptr(),
                    float(cap), float(q_scale), memory.data_ptr(), normalizer.data_ptr(), maximum.data_ptr(), slot_ids.data_ptr(),
-                   cu_rows.data_ptr(), y.data_ptr(), n_seq, heads, dk, dv, self._stream())
+                   cu_rows.data_ptr(), y.data_ptr(), n_seq, heads, dk, dv, chunk, n_chunks, ws.data_ptr() if ws is not None else None,
+                   self._stream())
         return y
 
     def pair_norm_mean(self, a, b, gain_a, gain_b, eps):
