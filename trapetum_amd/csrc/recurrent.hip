@@ -181,7 +181,6 @@ time_mix_scan_k(TimeMixArgs a) {
     float S[DK];
 #pragma unroll
     for (int i = 0; i < DK; i++) {                      // every lane reads an element that exists; what is none of S becomes zero
-        if (i % 16 == 0) __builtin_amdgcn_sched_barrier(0);
         const float x = MODE != TP_SCAN_LOCAL ? from[min(i, d - 1) * d + min(j, d - 1)] : 0.f;
         S[i] = (col && i < d) ? x : 0.f;
     }
@@ -358,7 +357,6 @@ matrix_memory_scan_k(MatrixMemoryArgs a) {
     float S[DK], nn[NR];
 #pragma unroll
     for (int i = 0; i < DK; i++) {                      // every lane reads an element that exists; what is none of S becomes zero
-        if (i % 16 == 0) __builtin_amdgcn_sched_barrier(0);
         const float x = MODE != TP_SCAN_LOCAL ? from[min(i, dk - 1) * dv + min(j, dv - 1)] : 0.f;
         S[i] = (col && i < dk) ? x : 0.f;
     }
