@@ -8,11 +8,13 @@
 //   head_norm_gate      every head's part of a row over its root mean square, times a gain, times sigmoid(g) or silu(g)
 //   weighted_sum        out = wa a + wb b
 //
-// Both scans run one wave for every (sequence, head, 64 value columns): a lane keeps one column of S in registers (all
-// key rows), the per-row vectors of a token (k, q or r, the decay) are formed one row a lane and reach the others through
-// LDS, where every lane reads the same four rows at a time (lane reads into scalar registers cost more: a token's few
-// hundred of them do not fit the scalar file), and the tokens of a sequence are taken in order, the next few tokens'
-// loads in flight while the present ones are worked on.  States, gates, decays and sums are float32; nothing is added across waves.
+// Both scans give 64 value columns of a (sequence, head) to one wave, or, for heads of 64 key rows and more, to a few waves
+// of a block that each keep a part of the rows: a lane keeps its wave's rows of one column of S in registers.  The per-row
+// vectors of a token (k, q or r, the decay) are formed one row a lane and reach the others through LDS, where every lane
+// reads the same four rows at a time (lane reads into scalar registers cost more: a token's few hundred of them do not
+// fit the scalar file).  The tokens of a sequence are taken in order, the next few tokens' loads in flight while the
+// present ones are worked on; a row of S goes on by itself, an output is a sum over rows whose parts meet in LDS once for
+// the tokens in flight.  States, gates, decays and sums are float32.
 #include "common.h"
 
 __device__ __forceinline__ float lane_value(float x, int lane) {
@@ -158,11 +160,16 @@ struct TimeMixArgs {
     int chunk, n_chunks; float* ws_state; float* ws_decay;      // [sequences n_chunks, H, d, d] and [sequences n_chunks, H, d]
 };
 
+// Key rows of a head that one wave keeps: heads of 64 rows and more are split over four waves of a block (a row of S
+// goes on by itself; only an output is a sum over rows, and the waves' parts of it meet in LDS once for the tokens in
+// flight), so that a state is read by four times the waves and a lane keeps a quarter of a column.
+#define TP_SCAN_SPLIT(DK) ((DK) >= 64 ? 4 : 1)
+
 template <typename T, int DK, int MODE>
-__global__ void __launch_bounds__(64)
+__global__ void __launch_bounds__(64 * TP_SCAN_SPLIT(DK))
 time_mix_scan_k(TimeMixArgs a) {
-    constexpr int NR = (DK + 63) / 64, AH = DK > 64 ? 2 : TP_SCAN_AHEAD;      // fewer tokens in flight where S takes most registers
-    const int h = blockIdx.y, lane = threadIdx.x, j = blockIdx.z * 64 + lane;
+    constexpr int NR = (DK + 63) / 64, AH = TP_SCAN_AHEAD, RS = TP_SCAN_SPLIT(DK), DKW = DK / RS;
+    const int h = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, j = blockIdx.z * 64 + lane, row0 = wave * DKW;
     const int seq = MODE == TP_SCAN_WHOLE ? blockIdx.x : blockIdx.x / a.n_chunks;
     const int d = a.d, HD = a.H * d;
     const bool col = j < d;
@@ -178,11 +185,11 @@ time_mix_scan_k(TimeMixArgs a) {
     float* st = a.state + ((size_t)a.slot_ids[seq] * a.H + h) * d * d;
     float* wst = MODE == TP_SCAN_WHOLE ? st : a.ws_state + ((size_t)blockIdx.x * a.H + h) * d * d;
     const float* from = MODE == TP_SCAN_FINAL ? wst : st;
-    float S[DK];
+    float S[DKW];                                       // rows row0 .. row0 + DKW - 1 of column j
 #pragma unroll
-    for (int i = 0; i < DK; i++) {                      // every lane reads an element that exists; what is none of S becomes zero
-        const float x = MODE != TP_SCAN_LOCAL ? from[min(i, d - 1) * d + min(j, d - 1)] : 0.f;
-        S[i] = (col && i < d) ? x : 0.f;
+    for (int i = 0; i < DKW; i++) {                     // every lane reads an element that exists; what is none of S becomes zero
+        const float x = MODE != TP_SCAN_LOCAL ? from[min(row0 + i, d - 1) * d + min(j, d - 1)] : 0.f;
+        S[i] = (col && row0 + i < d) ? x : 0.f;
     }
     float u[NR], w0[NR], fall[NR];                       // fall: the sum of the rows' log decays over the chunk
     load_rows<float, NR>(u, a.bonus + (size_t)h * d, d, lane, 1.f);
@@ -201,9 +208,12 @@ time_mix_scan_k(TimeMixArgs a) {
         }
     };
     // the per-row vectors of the tokens in flight, written a row a lane and read back by every lane, four rows a read
-    __shared__ __attribute__((aligned(16))) float stage[AH][3][DK];
+    __shared__ __attribute__((aligned(16))) float stage_all[RS][AH][3][DK];      // every wave's own copy
+    __shared__ float parts[2][RS][AH][64];               // the waves' parts of the outputs, for rounds in turn
+    float (*stage)[3][DK] = stage_all[wave];
+    int round = 0;
     fetch(begin, rr, kk, ww, vv);
-    for (int t0 = begin; t0 < end; t0 += AH) {
+    for (int t0 = begin; t0 < end; t0 += AH, round ^= 1) {
         float rn[AH][NR], kn[AH][NR], wn[AH][NR], vn[AH];
         fetch(t0 + AH, rn, kn, wn, vn);
         float bonus_dot[AH];
@@ -233,12 +243,12 @@ time_mix_scan_k(TimeMixArgs a) {
             outs[p] = 0.f;
             if (t0 + p < end) {
                 const float vj = vv[p];
-                const float4* R4 = (const float4*)stage[p][0];
-                const float4* K4 = (const float4*)stage[p][1];
-                const float4* W4 = (const float4*)stage[p][2];
+                const float4* R4 = (const float4*)(stage[p][0] + row0);
+                const float4* K4 = (const float4*)(stage[p][1] + row0);
+                const float4* W4 = (const float4*)(stage[p][2] + row0);
                 if (MODE == TP_SCAN_LOCAL) {
 #pragma unroll
-                    for (int i = 0; i < DK; i += 4) {
+                    for (int i = 0; i < DKW; i += 4) {
                         if (i % 16 == 0) __builtin_amdgcn_sched_barrier(0);      // the reads of sixteen rows at a time, not of all
                         const float4 k4 = K4[i / 4], w4 = W4[i / 4];
                         S[i] = __builtin_fmaf(w4.x, S[i], k4.x * vj);
@@ -247,9 +257,9 @@ time_mix_scan_k(TimeMixArgs a) {
                         S[i + 3] = __builtin_fmaf(w4.w, S[i + 3], k4.w * vj);
                     }
                 } else {
-                    float o0 = bonus_dot[p] * vj, o1 = 0.f, o2 = 0.f, o3 = 0.f;       // four sums: no FMA waits for the one before
+                    float o0 = wave == 0 ? bonus_dot[p] * vj : 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;       // four sums: no FMA waits for the one before
 #pragma unroll
-                    for (int i = 0; i < DK; i += 4) {
+                    for (int i = 0; i < DKW; i += 4) {
                         if (i % 16 == 0) __builtin_amdgcn_sched_barrier(0);      // the reads of sixteen rows at a time, not of all
                         const float4 r4 = R4[i / 4], k4 = K4[i / 4], w4 = W4[i / 4];
                         o0 = __builtin_fmaf(r4.x, S[i], o0);
@@ -268,9 +278,21 @@ time_mix_scan_k(TimeMixArgs a) {
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
-        if (MODE != TP_SCAN_LOCAL && col)
+        if (MODE != TP_SCAN_LOCAL) {
+            if (RS > 1) {                                // wave p adds the waves' parts of token p and stores it
+                static_assert(RS == 1 || RS == AH, "a wave for every token in flight");
 #pragma unroll
-            for (int p = 0; p < AH; p++) if (t0 + p < end) a.y[(size_t)(t0 + p) * HD + (size_t)h * d + j] = outs[p];
+                for (int p = 0; p < AH; p++) parts[round][wave][p][lane] = outs[p];
+                __syncthreads();
+                float sum = 0.f;
+#pragma unroll
+                for (int w = 0; w < RS; w++) sum += parts[round][w][wave][lane];
+                if (col && t0 + wave < end) a.y[(size_t)(t0 + wave) * HD + (size_t)h * d + j] = sum;
+            } else if (col) {
+#pragma unroll
+                for (int p = 0; p < AH; p++) if (t0 + p < end) a.y[(size_t)(t0 + p) * HD + (size_t)h * d + j] = outs[p];
+            }
+        }
 #pragma unroll
         for (int p = 0; p < AH; p++) {
             vv[p] = vn[p];
@@ -281,8 +303,8 @@ time_mix_scan_k(TimeMixArgs a) {
     float* to = MODE == TP_SCAN_LOCAL ? wst : st;
     if (col && (MODE != TP_SCAN_FINAL || last))
 #pragma unroll
-        for (int i = 0; i < DK; i++) if (i < d) to[i * d + j] = S[i];
-    if (MODE == TP_SCAN_LOCAL && blockIdx.z == 0)
+        for (int i = 0; i < DKW; i++) if (row0 + i < d) to[(row0 + i) * d + j] = S[i];
+    if (MODE == TP_SCAN_LOCAL && blockIdx.z == 0 && wave == 0)
 #pragma unroll
         for (int n = 0; n < NR; n++) if (lane + 64 * n < d) a.ws_decay[((size_t)blockIdx.x * a.H + h) * d + lane + 64 * n] = expf(fall[n]);
 }
@@ -328,14 +350,18 @@ struct MatrixMemoryArgs {
 
 __device__ __forceinline__ float log_sigmoid_f(float z) { return -(log1pf(expf(-fabsf(z))) + fmaxf(-z, 0.f)); }
 
-// One block for a (sequence, head) or a (chunk, head), a wave for every 64 value columns: every wave carries n and m
-// along (they are the same in all), reads them before any wave writes them back, and the first wave stores them at the
-// end.  A chunk run from nothing starts with m = -inf: its first row's maximum is its input gate, and nothing is kept.
+// One block for a (sequence, head) or a (chunk, head), a group of waves for every 64 value columns: every wave carries n
+// and m along (they are the same in all), reads them before any wave writes them back, and the first wave stores them at
+// the end.  A chunk run from nothing starts with m = -inf: its first row's maximum is its input gate, and nothing is kept.
+// The matrix memory's split: a block holds up to four groups of 64 value columns, each in MM_SPLIT waves
+#define TP_MM_SPLIT(DK) ((DK) >= 256 ? 2 : (DK) >= 64 ? 4 : 1)
+
 template <typename T, int DK, int MODE>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256 * TP_MM_SPLIT(DK))
 matrix_memory_scan_k(MatrixMemoryArgs a) {
-    constexpr int NR = (DK + 63) / 64, AH = DK > 64 ? 2 : TP_SCAN_AHEAD;      // fewer tokens in flight where S takes most registers
-    const int h = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, j = threadIdx.x;
+    constexpr int NR = (DK + 63) / 64, RS = TP_MM_SPLIT(DK), AH = RS > 1 ? 2 : TP_SCAN_AHEAD, DKW = DK / RS;
+    const int h = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, group = wave / RS, part = wave % RS;
+    const int j = group * 64 + lane, row0 = part * DKW;
     const int seq = MODE == TP_SCAN_WHOLE ? blockIdx.x : blockIdx.x / a.n_chunks;
     const int dk = a.dk, dv = a.dv, H = a.H;
     const bool col = j < dv;
@@ -354,11 +380,11 @@ matrix_memory_scan_k(MatrixMemoryArgs a) {
     float* wst = MODE == TP_SCAN_WHOLE ? st : a.ws_state + ((size_t)blockIdx.x * H + h) * ((size_t)dk * dv + dk);
     float* aux = MODE == TP_SCAN_WHOLE ? sn : a.ws_aux + ((size_t)blockIdx.x * H + h) * 4;
     const float* from = MODE == TP_SCAN_FINAL ? wst : st;
-    float S[DK], nn[NR];
+    float S[DKW], nn[NR];                               // rows row0 .. row0 + DKW - 1 of column j; all of n, a row a lane
 #pragma unroll
-    for (int i = 0; i < DK; i++) {                      // every lane reads an element that exists; what is none of S becomes zero
-        const float x = MODE != TP_SCAN_LOCAL ? from[min(i, dk - 1) * dv + min(j, dv - 1)] : 0.f;
-        S[i] = (col && i < dk) ? x : 0.f;
+    for (int i = 0; i < DKW; i++) {                     // every lane reads an element that exists; what is none of S becomes zero
+        const float x = MODE != TP_SCAN_LOCAL ? from[min(row0 + i, dk - 1) * dv + min(j, dv - 1)] : 0.f;
+        S[i] = (col && row0 + i < dk) ? x : 0.f;
     }
     float m = -INFINITY, fsum = 0.f;
     if (MODE == TP_SCAN_LOCAL) {
@@ -384,10 +410,12 @@ matrix_memory_scan_k(MatrixMemoryArgs a) {
         F = a.gates[(size_t)t * 2 * H + H + h];
     };
     // every wave's own copy of q and k of the tokens in flight, written a row a lane and read back by every lane
-    __shared__ __attribute__((aligned(16))) float stage_all[4][AH][2][DK];
+    __shared__ __attribute__((aligned(16))) float stage_all[4 * RS][AH][2][DK];
+    __shared__ float parts[2][4 * RS][AH][64];           // the waves' parts of the outputs, for rounds in turn
     float (*stage)[2][DK] = stage_all[wave];
+    int round = 0;
     fetch(begin, qq, kk, vv, gi, gf);
-    for (int t0 = begin; t0 < end; t0 += AH) {
+    for (int t0 = begin; t0 < end; t0 += AH, round ^= 1) {
         float qn[AH][NR], kn[AH][NR], vn[AH], gin, gfn;
         fetch(t0 + AH, qn, kn, vn, gin, gfn);
         const float li = a.cap * tanhf(gi / a.cap), lf = log_sigmoid_f(a.cap * tanhf(gf / a.cap));
@@ -404,24 +432,25 @@ matrix_memory_scan_k(MatrixMemoryArgs a) {
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        float outs[AH];                                  // stored together after the tokens: no branch of the lanes between them
+        float outs[AH], dens[AH];                        // stored together after the tokens: no branch of the lanes between them
 #pragma unroll
         for (int p = 0; p < AH; p++) {
             outs[p] = 0.f;
+            dens[p] = 1.f;
             if (t0 + p < end) {
                 const float i_t = lane_value(li, p), f_t = lane_value(lf, p);
                 const float m_new = fmaxf(f_t + m, i_t);
                 const float keep = expf(f_t + m - m_new), take = expf(i_t - m_new);
                 m = m_new;
                 const float tv = take * vv[p];
-                const float4* Q4 = (const float4*)stage[p][0];
-                const float4* K4 = (const float4*)stage[p][1];
+                const float4* Q4 = (const float4*)(stage[p][0] + row0);
+                const float4* K4 = (const float4*)(stage[p][1] + row0);
                 if (MODE == TP_SCAN_LOCAL) {
                     fsum += f_t;
 #pragma unroll
                     for (int n = 0; n < NR; n++) nn[n] = __builtin_fmaf(keep, nn[n], take * kk[p][n]);
 #pragma unroll
-                    for (int i = 0; i < DK; i += 4) {
+                    for (int i = 0; i < DKW; i += 4) {
                         if (i % 16 == 0) __builtin_amdgcn_sched_barrier(0);      // the reads of sixteen rows at a time, not of all
                         const float4 k4 = K4[i / 4];
                         S[i] = __builtin_fmaf(keep, S[i], k4.x * tv);
@@ -439,7 +468,7 @@ matrix_memory_scan_k(MatrixMemoryArgs a) {
                     const float den = fmaxf(fabsf(wave_sum(dot)), expf(-m)) + 1e-6f;
                     float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;                    // four sums: no FMA waits for the one before
 #pragma unroll
-                    for (int i = 0; i < DK; i += 4) {
+                    for (int i = 0; i < DKW; i += 4) {
                         if (i % 16 == 0) __builtin_amdgcn_sched_barrier(0);      // the reads of sixteen rows at a time, not of all
                         const float4 q4 = Q4[i / 4], k4 = K4[i / 4];
                         S[i] = __builtin_fmaf(keep, S[i], k4.x * tv);
@@ -451,16 +480,32 @@ matrix_memory_scan_k(MatrixMemoryArgs a) {
                         S[i + 3] = __builtin_fmaf(keep, S[i + 3], k4.w * tv);
                         o3 = __builtin_fmaf(q4.w, S[i + 3], o3);
                     }
-                    outs[p] = ((o0 + o1) + (o2 + o3)) / den;
+                    outs[p] = (o0 + o1) + (o2 + o3);
+                    dens[p] = den;
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
-        if (MODE != TP_SCAN_LOCAL && col)
+        if (MODE != TP_SCAN_LOCAL) {
+            if (RS > 1) {                                // a group's first wave adds the parts of its waves
 #pragma unroll
-            for (int p = 0; p < AH; p++) if (t0 + p < end) a.y[((size_t)(t0 + p) * H + h) * dv + j] = outs[p];
+                for (int p = 0; p < AH; p++) parts[round][wave][p][lane] = outs[p];
+                __syncthreads();
+                if (part == 0)
+#pragma unroll
+                    for (int p = 0; p < AH; p++) {
+                        float sum = 0.f;
+#pragma unroll
+                        for (int w = 0; w < RS; w++) sum += parts[round][group * RS + w][p][lane];
+                        outs[p] = sum;
+                    }
+            }
+            if (col && part == 0)
+#pragma unroll
+                for (int p = 0; p < AH; p++) if (t0 + p < end) a.y[((size_t)(t0 + p) * H + h) * dv + j] = outs[p] / dens[p];
+        }
         gi = gin; gf = gfn;
 #pragma unroll
         for (int p = 0; p < AH; p++) {
@@ -474,7 +519,7 @@ matrix_memory_scan_k(MatrixMemoryArgs a) {
     float* to_n = MODE == TP_SCAN_LOCAL ? wst + (size_t)dk * dv : sn;
     if (col)
 #pragma unroll
-        for (int i = 0; i < DK; i++) if (i < dk) to[i * dv + j] = S[i];
+        for (int i = 0; i < DKW; i++) if (row0 + i < dk) to[(row0 + i) * dv + j] = S[i];
     if (wave == 0) {
 #pragma unroll
         for (int n = 0; n < NR; n++) if (lane + 64 * n < dk) to_n[lane + 64 * n] = nn[n];
@@ -565,7 +610,7 @@ extern "C" int tp_time_mix_scan(const void* r, long r_stride, const void* k, lon
     dim3 grid(n_seq, H, tp_cdiv(d, 64)), chunk_grid(n_seq * (chunk > 0 ? n_chunks : 1), H, tp_cdiv(d, 64)), carry_grid(n_seq, H, tp_cdiv(d * d, 256));
     hipStream_t s = (hipStream_t)stream;
     if (dtype != TP_BF16 && dtype != TP_F32) return tp_fail("time_mix_scan: unknown dtype %d", dtype);
-#define TP_LAUNCH(DK) TP_SCAN_MODES(time_mix_scan_k, (time_mix_carry_k<<<carry_grid, 256, 0, s>>>(state, slot_ids, cu_rows, workspace, ws_decay, H, d, chunk, n_chunks)), DK, grid, chunk_grid, 64)
+#define TP_LAUNCH(DK) TP_SCAN_MODES(time_mix_scan_k, (time_mix_carry_k<<<carry_grid, 256, 0, s>>>(state, slot_ids, cu_rows, workspace, ws_decay, H, d, chunk, n_chunks)), DK, grid, chunk_grid, 64 * TP_SCAN_SPLIT(DK))
     TP_SCAN_SIZES(TP_LAUNCH, d);
 #undef TP_LAUNCH
     return tp_check_launch("time_mix_scan");
@@ -592,10 +637,10 @@ extern "C" int tp_matrix_memory_scan(const void* q, long q_stride, const void* k
     MatrixMemoryArgs a{q, q_stride, k, k_stride, v, v_stride, gates, cap, q_scale, memory, normalizer, maximum, slot_ids, cu_rows, y, H, dk, dv,
                        chunk, n_chunks, workspace, ws_aux};
     dim3 grid(n_seq, H), chunk_grid(n_seq * (chunk > 0 ? n_chunks : 1), H), carry_grid(n_seq, H, tp_cdiv(dk * dv + dk, 256));
-    const int threads = 64 * tp_cdiv(dv, 64);
+    const int threads = 64 * tp_cdiv(dv, 64);            // times the waves a group of columns is split over
     hipStream_t s = (hipStream_t)stream;
     if (dtype != TP_BF16 && dtype != TP_F32) return tp_fail("matrix_memory_scan: unknown dtype %d", dtype);
-#define TP_LAUNCH(DK) TP_SCAN_MODES(matrix_memory_scan_k, (matrix_memory_carry_k<<<carry_grid, 256, 0, s>>>(memory, normalizer, maximum, slot_ids, cu_rows, workspace, ws_aux, H, dk, dv, chunk, n_chunks)), DK, grid, chunk_grid, threads)
+#define TP_LAUNCH(DK) TP_SCAN_MODES(matrix_memory_scan_k, (matrix_memory_carry_k<<<carry_grid, 256, 0, s>>>(memory, normalizer, maximum, slot_ids, cu_rows, workspace, ws_aux, H, dk, dv, chunk, n_chunks)), DK, grid, chunk_grid, threads * TP_MM_SPLIT(DK))
     TP_SCAN_SIZES(TP_LAUNCH, dk);
 #undef TP_LAUNCH
     return tp_check_launch("matrix_memory_scan");
