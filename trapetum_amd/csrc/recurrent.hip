@@ -196,27 +196,32 @@ time_mix_scan_k(TimeMixArgs a) {
     load_rows<float, NR>(w0, a.w0 + (size_t)h * d, d, lane, 1.f);
 #pragma unroll
     for (int n = 0; n < NR; n++) fall[n] = 0.f;
-    float rr[AH][NR], kk[AH][NR], ww[AH][NR], vv[AH];
+    // the block's first wave forms the per-row vectors of the tokens in flight for all its waves
+    const bool stager = RS == 1 || wave == 0;
+    float rr[AH][NR] = {}, kk[AH][NR] = {}, ww[AH][NR] = {}, vv[AH];
     auto fetch = [&](int t0, float (&R)[AH][NR], float (&K)[AH][NR], float (&W)[AH][NR], float (&V)[AH]) {
 #pragma unroll
         for (int p = 0; p < AH; p++) {
             const int t = min(t0 + p, end - 1);          // past the end: a row that exists, never used
-            if (MODE != TP_SCAN_LOCAL) load_rows<T, NR>(R[p], (const T*)a.r + (size_t)t * a.r_stride + (size_t)h * d, d, lane, 1.f);
-            load_rows<T, NR>(K[p], (const T*)a.k + (size_t)t * a.k_stride + (size_t)h * d, d, lane, 1.f);
-            load_rows<float, NR>(W[p], a.log_rate + (size_t)t * HD + (size_t)h * d, d, lane, 1.f);
+            if (stager) {
+                if (MODE != TP_SCAN_LOCAL) load_rows<T, NR>(R[p], (const T*)a.r + (size_t)t * a.r_stride + (size_t)h * d, d, lane, 1.f);
+                load_rows<T, NR>(K[p], (const T*)a.k + (size_t)t * a.k_stride + (size_t)h * d, d, lane, 1.f);
+                load_rows<float, NR>(W[p], a.log_rate + (size_t)t * HD + (size_t)h * d, d, lane, 1.f);
+            }
             V[p] = col ? ld_f32((const T*)a.v + (size_t)t * a.v_stride + (size_t)h * d + j) : 0.f;
         }
     };
     // the per-row vectors of the tokens in flight, written a row a lane and read back by every lane, four rows a read
-    __shared__ __attribute__((aligned(16))) float stage_all[RS][AH][3][DK];      // every wave's own copy
+    __shared__ __attribute__((aligned(16))) float stage_all[2][AH][3][DK];       // for rounds in turn
     __shared__ float parts[2][RS][AH][64];               // the waves' parts of the outputs, for rounds in turn
-    float (*stage)[3][DK] = stage_all[wave];
     int round = 0;
     fetch(begin, rr, kk, ww, vv);
     for (int t0 = begin; t0 < end; t0 += AH, round ^= 1) {
-        float rn[AH][NR], kn[AH][NR], wn[AH][NR], vn[AH];
+        float (*stage)[3][DK] = stage_all[round];
+        float rn[AH][NR] = {}, kn[AH][NR] = {}, wn[AH][NR] = {}, vn[AH];
         fetch(t0 + AH, rn, kn, wn, vn);
-        float bonus_dot[AH];
+        float bonus_dot[AH] = {};
+        if (stager)
 #pragma unroll
         for (int p = 0; p < AH; p++) {
             float dot = 0.f;
@@ -234,9 +239,12 @@ time_mix_scan_k(TimeMixArgs a) {
             }
             bonus_dot[p] = MODE != TP_SCAN_LOCAL ? wave_sum(dot) : 0.f;     // the present token's bonus: sum_i r_i u_i k_i
         }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        if (RS > 1) __syncthreads();
+        else {
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        }
         float outs[AH];                                  // stored together after the tokens: no branch of the lanes between them
 #pragma unroll
         for (int p = 0; p < AH; p++) {
@@ -396,59 +404,80 @@ matrix_memory_scan_k(MatrixMemoryArgs a) {
     }
     __syncthreads();
     // lane p of a group of tokens forms token p's two gates; the others read them from it
-    float qq[AH][NR], kk[AH][NR], vv[AH], gi, gf;
+    // the block's first wave forms q and k of the tokens in flight for all its waves, carries n and forms the denominators
+    const bool stager = wave == 0;
+    float qq[AH][NR] = {}, kk[AH][NR] = {}, vv[AH], gi, gf;
     auto fetch = [&](int t0, float (&Q)[AH][NR], float (&K)[AH][NR], float (&V)[AH], float& I, float& F) {
 #pragma unroll
         for (int p = 0; p < AH; p++) {
             const int t = min(t0 + p, end - 1);
-            if (MODE != TP_SCAN_LOCAL) load_rows<T, NR>(Q[p], (const T*)a.q + (size_t)t * a.q_stride + (size_t)h * dk, dk, lane, a.q_scale);
-            load_rows<T, NR>(K[p], (const T*)a.k + (size_t)t * a.k_stride + (size_t)h * dk, dk, lane, 1.f);
+            if (stager) {
+                if (MODE != TP_SCAN_LOCAL) load_rows<T, NR>(Q[p], (const T*)a.q + (size_t)t * a.q_stride + (size_t)h * dk, dk, lane, a.q_scale);
+                load_rows<T, NR>(K[p], (const T*)a.k + (size_t)t * a.k_stride + (size_t)h * dk, dk, lane, 1.f);
+            }
             V[p] = col ? ld_f32((const T*)a.v + (size_t)t * a.v_stride + (size_t)h * dv + j) : 0.f;
         }
         const int t = min(t0 + min(lane, AH - 1), end - 1);
         I = a.gates[(size_t)t * 2 * H + h];
         F = a.gates[(size_t)t * 2 * H + H + h];
     };
-    // every wave's own copy of q and k of the tokens in flight, written a row a lane and read back by every lane
-    __shared__ __attribute__((aligned(16))) float stage_all[4 * RS][AH][2][DK];
+    // q and k of the tokens in flight, written a row a lane by the first wave and read back by every lane; for rounds in turn
+    __shared__ __attribute__((aligned(16))) float stage_all[2][AH][2][DK];
+    __shared__ float dens_all[2][AH];
     __shared__ float parts[2][4 * RS][AH][64];           // the waves' parts of the outputs, for rounds in turn
-    float (*stage)[2][DK] = stage_all[wave];
     int round = 0;
     fetch(begin, qq, kk, vv, gi, gf);
     for (int t0 = begin; t0 < end; t0 += AH, round ^= 1) {
-        float qn[AH][NR], kn[AH][NR], vn[AH], gin, gfn;
+        float (*stage)[2][DK] = stage_all[round];
+        float qn[AH][NR] = {}, kn[AH][NR] = {}, vn[AH], gin, gfn;
         fetch(t0 + AH, qn, kn, vn, gin, gfn);
         const float li = a.cap * tanhf(gi / a.cap), lf = log_sigmoid_f(a.cap * tanhf(gf / a.cap));
+        // what the gates make of m, token after token: every wave for itself
+        float keeps[AH], takes[AH], floors[AH];
 #pragma unroll
-        for (int p = 0; p < AH; p++)
+        for (int p = 0; p < AH; p++) {
+            keeps[p] = 1.f; takes[p] = 0.f; floors[p] = 1.f;
+            if (t0 + p < end) {
+                const float i_t = lane_value(li, p), f_t = lane_value(lf, p);
+                const float m_new = fmaxf(f_t + m, i_t);
+                keeps[p] = expf(f_t + m - m_new);
+                takes[p] = expf(i_t - m_new);
+                m = m_new;
+                floors[p] = expf(-m);
+                if (MODE == TP_SCAN_LOCAL) fsum += f_t;
+            }
+        }
+        if (stager)
 #pragma unroll
-            for (int n = 0; n < NR; n++) {
-                const int row = lane + 64 * n;
-                if (row < DK) {
-                    if (MODE != TP_SCAN_LOCAL) stage[p][0][row] = qq[p][n];
-                    stage[p][1][row] = kk[p][n];
+            for (int p = 0; p < AH; p++) {
+                float dot = 0.f;
+#pragma unroll
+                for (int n = 0; n < NR; n++) {
+                    const int row = lane + 64 * n;
+                    if (t0 + p < end) nn[n] = __builtin_fmaf(keeps[p], nn[n], takes[p] * kk[p][n]);
+                    if (MODE != TP_SCAN_LOCAL) dot = __builtin_fmaf(nn[n], qq[p][n], dot);
+                    if (row < DK) {
+                        if (MODE != TP_SCAN_LOCAL) stage[p][0][row] = qq[p][n];
+                        stage[p][1][row] = kk[p][n];
+                    }
+                }
+                if (MODE != TP_SCAN_LOCAL) {
+                    const float den = fmaxf(fabsf(wave_sum(dot)), floors[p]) + 1e-6f;
+                    if (lane == 0) dens_all[round][p] = den;
                 }
             }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        __syncthreads();
         float outs[AH], dens[AH];                        // stored together after the tokens: no branch of the lanes between them
 #pragma unroll
         for (int p = 0; p < AH; p++) {
             outs[p] = 0.f;
-            dens[p] = 1.f;
+            dens[p] = MODE != TP_SCAN_LOCAL ? dens_all[round][p] : 1.f;
             if (t0 + p < end) {
-                const float i_t = lane_value(li, p), f_t = lane_value(lf, p);
-                const float m_new = fmaxf(f_t + m, i_t);
-                const float keep = expf(f_t + m - m_new), take = expf(i_t - m_new);
-                m = m_new;
-                const float tv = take * vv[p];
+                const float keep = keeps[p];
+                const float tv = takes[p] * vv[p];
                 const float4* Q4 = (const float4*)(stage[p][0] + row0);
                 const float4* K4 = (const float4*)(stage[p][1] + row0);
                 if (MODE == TP_SCAN_LOCAL) {
-                    fsum += f_t;
-#pragma unroll
-                    for (int n = 0; n < NR; n++) nn[n] = __builtin_fmaf(keep, nn[n], take * kk[p][n]);
 #pragma unroll
                     for (int i = 0; i < DKW; i += 4) {
                         if (i % 16 == 0) __builtin_amdgcn_sched_barrier(0);      // the reads of sixteen rows at a time, not of all
@@ -459,13 +488,6 @@ matrix_memory_scan_k(MatrixMemoryArgs a) {
                         S[i + 3] = __builtin_fmaf(keep, S[i + 3], k4.w * tv);
                     }
                 } else {
-                    float dot = 0.f;
-#pragma unroll
-                    for (int n = 0; n < NR; n++) {
-                        nn[n] = __builtin_fmaf(keep, nn[n], take * kk[p][n]);
-                        dot = __builtin_fmaf(nn[n], qq[p][n], dot);
-                    }
-                    const float den = fmaxf(fabsf(wave_sum(dot)), expf(-m)) + 1e-6f;
                     float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;                    // four sums: no FMA waits for the one before
 #pragma unroll
                     for (int i = 0; i < DKW; i += 4) {
@@ -481,7 +503,6 @@ matrix_memory_scan_k(MatrixMemoryArgs a) {
                         o3 = __builtin_fmaf(q4.w, S[i + 3], o3);
                     }
                     outs[p] = (o0 + o1) + (o2 + o3);
-                    dens[p] = den;
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
