@@ -10,9 +10,9 @@
 //
 // Both scans give 64 value columns of a (sequence, head) to one wave, or, for heads of 64 key rows and more, to a few waves
 // of a block that each keep a part of the rows: a lane keeps its wave's rows of one column of S in registers.  The per-row
-// vectors of a token (k, q or r, the decay) are formed one row a lane and reach the others through LDS, where every lane
-// reads the same four rows at a time (lane reads into scalar registers cost more: a token's few hundred of them do not
-// fit the scalar file).  The tokens of a sequence are taken in order, the next few tokens' loads in flight while the
+// vectors of a token (k, q or r, the decay) are formed one row a lane by the block's first wave and reach all lanes through
+// LDS, where every lane reads the same four rows at a time (lane reads into scalar registers cost more: a token's few
+// hundred of them do not fit the scalar file).  The tokens of a sequence are taken in order, the next few tokens' loads in flight while the
 // present ones are worked on; a row of S goes on by itself, an output is a sum over rows whose parts meet in LDS once for
 // the tokens in flight.  States, gates, decays and sums are float32.
 #include "common.h"
