@@ -49,16 +49,18 @@ class GroupPages:
     """Pages of one group of layers: a pool and each slot's page list.
 
     `rows_cap`: None if a sequence keeps every row, else the number of rows of its
-    ring (position p lives in ring row p % rows_cap)."""
+    ring (position p lives in ring row p % rows_cap).  `every`: tokens per row (a row exists once its last token does)."""
 
-    def __init__(self, n_pages, page_size, rows_cap, name):
+    def __init__(self, n_pages, page_size, rows_cap, name, every=1):
         self.page_size = page_size
         self.rows_cap = rows_cap
+        self.every = every
         self.name = name
         self.pool = FreeList(n_pages, f"page of cache group '{name}'")
         self.lists = {}                               # slot -> [page ids]
 
     def rows_needed(self, length):
+        length //= self.every
         return length if self.rows_cap is None else min(length, self.rows_cap)
 
     def pages_needed(self, length):

@@ -36,14 +36,18 @@ class TokenSpec:
     """What a mixer keeps of every token: named tensors, each of a fixed shape, in the engine's activation dtype."""
     tensors: tuple                      # ((name, shape), ...): hashable, in the mixer's order
     window: Optional[int] = None        # None: every token is kept
+    every: int = 1                      # one row per `every` tokens: row b belongs to the positions b * every .. b * every + every - 1
+                                        # and exists once the last of them does (a summary of a block of tokens)
 
     @staticmethod
-    def of(window=None, **tensors):
+    def of(window=None, every=1, **tensors):
         """TokenSpec.of(window, k=(kv_heads, head_dim), v=(kv_heads, head_dim))"""
         for name, shape in tensors.items():
             if not shape or any(int(n) <= 0 for n in shape):
                 raise CacheError(f"per-token tensor '{name}' needs a shape of positive sizes, found {shape!r}")
-        return TokenSpec(tuple((name, tuple(int(n) for n in shape)) for name, shape in tensors.items()), window)
+        if int(every) < 1 or (int(every) > 1 and window is not None):
+            raise CacheError(f"a row per {every} tokens: the number must be positive, and such rows are kept of all tokens, not of a window")
+        return TokenSpec(tuple((name, tuple(int(n) for n in shape)) for name, shape in tensors.items()), window, int(every))
 
     def shape_of(self, name):
         for n, shape in self.tensors:
@@ -93,7 +97,9 @@ class _TokenGroup:
         if spec.window is not None and spec.window < max_context:
             rows_cap = -(-spec.window // page_size) * page_size
             n_pages = min(n_pages, max_slots * (rows_cap // page_size))      # a ring never grows beyond its rows
-        self.pages = GroupPages(n_pages, page_size, rows_cap, name)
+        if spec.every > 1:                                                   # whole pages of rows, and a last page per sequence
+            n_pages = min(n_pages, -(-n_pages // spec.every) + max_slots)
+        self.pages = GroupPages(n_pages, page_size, rows_cap, name, every=spec.every)
         self.spare_page = n_pages                                          # the pool's last page, never handed out
         self.pools = {}
         for tname, shape in spec.tensors:
@@ -117,9 +123,11 @@ class ModelCache:
     max_context: longest single sequence.
     """
 
-    def __init__(self, entry_specs, max_tokens, max_context, max_slots, page_size, dtype, device, entry_states=None):
+    def __init__(self, entry_specs, max_tokens, max_context, max_slots, page_size, dtype, device, entry_states=None, entry_tokens=None):
         """entry_states: for every schedule entry, {name: StateSpec} of states it keeps beside its mixer's cache (what a
-        block's own operations carry from step to step); a run that reads another run's cache still has its own."""
+        block's own operations carry from step to step); a run that reads another run's cache still has its own.
+        entry_tokens: for every schedule entry, {name: TokenSpec} of further paged tensors it keeps by name (rows at
+        another rate than its mixer's cache: one per block of tokens)."""
         if page_size <= 0 or page_size % 16:
             raise CacheError(f"page size {page_size} must be a positive multiple of 16")
         self.page_size = page_size
@@ -134,12 +142,15 @@ class ModelCache:
         for entry, spec in enumerate(entry_specs):
             if spec is not None:
                 keyed.setdefault(spec, []).append(entry)
+        def token_group(spec, entries):
+            name = f"tokens{len(self.token_groups)}:" + ("all" if spec.window is None else f"window{spec.window}") + \
+                (f"/{spec.every}" if spec.every > 1 else "")
+            g = _TokenGroup(spec, entries, n_pages, max_slots, page_size, max_context, dtype, device, name)
+            self.token_groups.append(g)
+            return g, len(self.token_groups) - 1
         for spec, entries in keyed.items():
             if isinstance(spec, TokenSpec):
-                name = f"tokens{len(self.token_groups)}:" + ("all" if spec.window is None else f"window{spec.window}")
-                g = _TokenGroup(spec, entries, n_pages, max_slots, page_size, max_context, dtype, device, name)
-                gi = len(self.token_groups)
-                self.token_groups.append(g)
+                g, gi = token_group(spec, entries)
             elif isinstance(spec, StateSpec):
                 g = _StateGroup(spec, entries, max_slots, dtype, device)
                 gi = len(self.state_groups)
@@ -148,6 +159,17 @@ class ModelCache:
                 raise CacheError(f"schedule entry declares an unknown cache need: {spec!r}")
             for i, entry in enumerate(entries):
                 self._site_of[entry] = CacheSite(spec, gi, i, g)
+        self._named_sites = {}
+        keyed = {}
+        for entry, named in enumerate(entry_tokens or ()):
+            for name, spec in (named or {}).items():
+                if not isinstance(spec, TokenSpec):
+                    raise CacheError(f"schedule entry {entry} declares paged tensors '{name}' as {spec!r}: not a TokenSpec")
+                keyed.setdefault(spec, []).append((entry, name))
+        for spec, owners in keyed.items():
+            g, gi = token_group(spec, [e for e, _ in owners])
+            for i, owner in enumerate(owners):
+                self._named_sites[owner] = CacheSite(spec, gi, i, g)
         self._named_states = {}
         keyed = {}
         for entry, states in enumerate(entry_states or ()):
@@ -171,6 +193,12 @@ class ModelCache:
         if (entry, name) not in self._named_states:
             raise CacheError(f"schedule entry {entry} declared no state '{name}'")
         return self._named_states[(entry, name)]
+
+    def entry_site(self, entry, name):
+        """The paged tensors an entry declared by name, as a site like the one of its mixer's cache."""
+        if (entry, name) not in self._named_sites:
+            raise CacheError(f"schedule entry {entry} declared no paged tensors '{name}'")
+        return self._named_sites[(entry, name)]
 
     # --- what the engine uses ---------------------------------------------------------
     def acquire(self):

@@ -681,3 +681,57 @@ extern "C" int tp_gated_act(const float* y, void* out, int dtype, int M, int I, 
     else return tp_fail("gated_act: unknown dtype %d", dtype);
     return tp_check_launch("gated_act");
 }
+
+// ---- out = act(rows + bias): a dense feed-forward's first product with its bias and activation ---------------------
+// rows float32 or bf16 [M, N], out in its own dtype; act 0: none, 1: the exact gelu, x Phi(x) = 0.5 x (1 + erf(x / sqrt 2)).
+enum { TP_BIAS_NONE = 0, TP_BIAS_GELU_ERF = 1 };
+template <typename TI, typename TO>
+__global__ void bias_act_k(const TI* __restrict__ rows, const float* __restrict__ bias, TO* __restrict__ out, long total, int N, int act) {
+    for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+        float y = ld_f32(rows + i) + (bias ? bias[i % N] : 0.f);
+        if (act == TP_BIAS_GELU_ERF) y = 0.5f * y * (1.f + erff(y * 0.70710678118654752f));
+        st_f32(out + i, y);
+    }
+}
+
+extern "C" int tp_bias_act(const void* rows, int in_dtype, const float* bias, void* out, int out_dtype, int M, int N, int act, void* stream) {
+    TP_REQUIRE(rows && out && M > 0 && N > 0, "bias_act: empty shape M=%d N=%d", M, N);
+    TP_REQUIRE(act == TP_BIAS_NONE || act == TP_BIAS_GELU_ERF, "bias_act: unknown activation %d", act);
+    const long total = (long)M * N;
+    long blocks = (total + 255) / 256;
+    if (blocks > 8192) blocks = 8192;
+    hipStream_t s = (hipStream_t)stream;
+    if (in_dtype == TP_F32 && out_dtype == TP_F32) bias_act_k<float, float><<<(unsigned)blocks, 256, 0, s>>>((const float*)rows, bias, (float*)out, total, N, act);
+    else if (in_dtype == TP_F32 && out_dtype == TP_BF16) bias_act_k<float, bf16_t><<<(unsigned)blocks, 256, 0, s>>>((const float*)rows, bias, (bf16_t*)out, total, N, act);
+    else if (in_dtype == TP_BF16 && out_dtype == TP_BF16) bias_act_k<bf16_t, bf16_t><<<(unsigned)blocks, 256, 0, s>>>((const bf16_t*)rows, bias, (bf16_t*)out, total, N, act);
+    else return tp_fail("bias_act: no kernel from dtype %d to dtype %d", in_dtype, out_dtype);
+    return tp_check_launch("bias_act");
+}
+
+// ---- x[r, h, :] *= sigmoid(g[r, h]): a gate per head (or, with one head, per row) --------------------------------------
+template <typename T, typename TG>
+__global__ void __launch_bounds__(256)
+mul_sigmoid_heads_k(T* __restrict__ x, long x_stride, const TG* __restrict__ g, long g_stride, int M, int H, int per) {
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    const long C = (long)H * per;
+    if (i >= (long)M * C) return;
+    const long r = i / C, c = i - r * C;
+    T* xp = x + r * x_stride + c;
+    const float gv = ld_f32(g + r * g_stride + c / per);
+    st_f32(xp, ld_f32(xp) / (1.f + expf(-gv)));
+}
+
+extern "C" int tp_mul_sigmoid_heads(void* x, long x_stride, int x_dtype, const void* g, long g_stride, int g_dtype, int M, int H, int per, void* stream) {
+    TP_REQUIRE(M > 0 && H > 0 && per > 0 && x && g, "mul_sigmoid_heads: empty shape or null operand (M=%d H=%d per=%d)", M, H, per);
+    hipStream_t s = (hipStream_t)stream;
+    const long blocks = ((long)M * H * per + 255) / 256;
+    TP_REQUIRE(blocks <= 0x7fffffffL, "mul_sigmoid_heads: %ld blocks exceed one launch", blocks);
+#define TP_MSH(T, TG) mul_sigmoid_heads_k<T, TG><<<(unsigned)blocks, 256, 0, s>>>((T*)x, x_stride, (const TG*)g, g_stride, M, H, per)
+    if (x_dtype == TP_F32 && g_dtype == TP_F32) TP_MSH(float, float);
+    else if (x_dtype == TP_BF16 && g_dtype == TP_F32) TP_MSH(bf16_t, float);
+    else if (x_dtype == TP_BF16 && g_dtype == TP_BF16) TP_MSH(bf16_t, bf16_t);
+    else if (x_dtype == TP_F32 && g_dtype == TP_BF16) TP_MSH(float, bf16_t);
+    else return tp_fail("mul_sigmoid_heads: unknown dtypes %d, %d", x_dtype, g_dtype);
+#undef TP_MSH
+    return tp_check_launch("mul_sigmoid_heads");
+}

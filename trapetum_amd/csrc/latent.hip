@@ -15,7 +15,7 @@ latent_prepare_k(const T* __restrict__ proj, long proj_stride, int H, int dn, in
                  const float* __restrict__ gain, float eps, const float* __restrict__ inv_freq, int rot,
                  const int* __restrict__ row_seq, const int* __restrict__ row_pos, const int* __restrict__ new_len,
                  const int* __restrict__ table, int table_w, T* __restrict__ pool, int page, int rows_cap,
-                 T* __restrict__ q, T* __restrict__ mine, int own) {
+                 T* __restrict__ q, T* __restrict__ mine, int own, const T* __restrict__ tail_rows, long tail_stride) {
     extern __shared__ float cs[];                        // [rot / 2] cosines, [rot / 2] sines
     __shared__ float red[16];
     const int r = blockIdx.x, pos = row_pos[r], half = rot / 2, row = dr + R;
@@ -37,7 +37,7 @@ latent_prepare_k(const T* __restrict__ proj, long proj_stride, int H, int dn, in
         st_f32(qr + (size_t)h * row + e, y);
     }
     if (!own) return;
-    const T* tail = pr + (size_t)H * (dr + dn);
+    const T* tail = tail_rows ? tail_rows + (size_t)r * tail_stride : pr + (size_t)H * (dr + dn);     // a product of its own, or the row's end
     T* dst = nullptr;                                    // the row's place in the cache
     if (table) {
         const int seq = row_seq[r];
@@ -74,12 +74,13 @@ extern "C" int tp_latent_prepare(const void* proj, long proj_stride, int dtype, 
                                  const float* gain, float eps, const float* inv_freq, int rot,
                                  const int* row_seq, const int* row_pos, const int* new_len,
                                  const int* table, int table_w, void* pool, int page, int rows_cap,
-                                 void* q, void* mine, int own, void* stream) {
+                                 void* q, void* mine, int own, const void* tail, long tail_stride, void* stream) {
     TP_REQUIRE(M > 0 && H > 0 && dn >= 0 && dr >= 0 && R > 0, "latent_prepare: empty shape M=%d H=%d dn=%d dr=%d R=%d", M, H, dn, dr, R);
     TP_REQUIRE(proj && q && row_pos, "latent_prepare: a null operand");
     TP_REQUIRE(rot >= 0 && rot <= dr && rot % 2 == 0, "latent_prepare: %d turning elements must be even and at most the rotated part's %d", rot, dr);
     TP_REQUIRE(rot == 0 || inv_freq, "latent_prepare: a rotation needs its frequency table");
-    TP_REQUIRE(proj_stride >= (long)H * (dr + dn) + (own ? dr + R : 0), "latent_prepare: rows of %ld elements are too short", proj_stride);
+    TP_REQUIRE(proj_stride >= (long)H * (dr + dn) + (own && !tail ? dr + R : 0), "latent_prepare: rows of %ld elements are too short", proj_stride);
+    TP_REQUIRE(!tail || (own && tail_stride >= dr + R), "latent_prepare: the key part and latent as rows of their own need %d elements a row", dr + R);
     TP_REQUIRE(!own || (mine && gain && row_seq && new_len), "latent_prepare: a layer with a latent of its own needs its gain and the rows' output");
     TP_REQUIRE(!table || (pool && page > 0 && table_w > 0), "latent_prepare: a page table without a cache pool");
     if (!table) { page = 1; rows_cap = 0; }
@@ -89,10 +90,10 @@ extern "C" int tp_latent_prepare(const void* proj, long proj_stride, int dtype, 
     const size_t lds = (size_t)rot * sizeof(float);
     if (dtype == TP_BF16)
         latent_prepare_k<bf16_t><<<M, 256, lds, s>>>((const bf16_t*)proj, proj_stride, H, dn, dr, R, gain, eps, inv_freq, rot, row_seq, row_pos,
-            new_len, table, table_w, (bf16_t*)pool, page, rows_cap, (bf16_t*)q, (bf16_t*)mine, own);
+            new_len, table, table_w, (bf16_t*)pool, page, rows_cap, (bf16_t*)q, (bf16_t*)mine, own, (const bf16_t*)tail, tail_stride);
     else if (dtype == TP_F32)
         latent_prepare_k<float><<<M, 256, lds, s>>>((const float*)proj, proj_stride, H, dn, dr, R, gain, eps, inv_freq, rot, row_seq, row_pos,
-            new_len, table, table_w, (float*)pool, page, rows_cap, (float*)q, (float*)mine, own);
+            new_len, table, table_w, (float*)pool, page, rows_cap, (float*)q, (float*)mine, own, (const float*)tail, tail_stride);
     else return tp_fail("latent_prepare: unknown dtype %d", dtype);
     return tp_check_launch("latent_prepare");
 }

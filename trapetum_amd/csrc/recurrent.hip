@@ -26,10 +26,10 @@ enum { TP_GATE_SIGMOID = 0, TP_GATE_SILU = 1 };
 
 // ---- the mixes of a row with the row before it -----------------------------------------------------------------------
 // grid (rows, blocks of 256 channels).  state [slots, D] float32: the last row of the sequence's step before.
-template <typename T>
+template <typename T, typename TO>
 __global__ void __launch_bounds__(256)
 shift_mix_k(const T* __restrict__ x, const float* __restrict__ mu, float* __restrict__ state, const int* __restrict__ slot_ids,
-            const int* __restrict__ cu_rows, const int* __restrict__ row_seq, T* __restrict__ out, int M, int D, int n_mix, int save) {
+            const int* __restrict__ cu_rows, const int* __restrict__ row_seq, TO* __restrict__ out, int M, int D, int n_mix, int save) {
     const int r = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
     if (c >= D) return;
     const int seq = row_seq[r];
@@ -50,20 +50,22 @@ shift_save_k(const T* __restrict__ x, float* __restrict__ state, const int* __re
     state[(size_t)slot_ids[seq] * D + c] = ld_f32(x + (size_t)(cu_rows[seq + 1] - 1) * D + c);
 }
 
+// out_dtype: the mixes' dtype; it may be narrower than the rows' (float32 rows of a norm, mixes in bfloat16: one rounding)
 extern "C" int tp_shift_mix(const void* x, int dtype, const float* mu, int n_mix, float* state, const int* slot_ids, const int* cu_rows,
-                            const int* row_seq, void* out, int M, int n_seq, int D, int one_row_each, void* stream) {
+                            const int* row_seq, void* out, int out_dtype, int M, int n_seq, int D, int one_row_each, void* stream) {
     TP_REQUIRE(M > 0 && n_seq > 0 && D > 0 && n_mix > 0, "shift_mix: empty shape rows=%d sequences=%d channels=%d mixes=%d", M, n_seq, D, n_mix);
     TP_REQUIRE(x && mu && state && slot_ids && cu_rows && row_seq && out, "shift_mix: null operand");
     TP_REQUIRE(!one_row_each || M == n_seq, "shift_mix: one row each, but %d rows of %d sequences", M, n_seq);
     hipStream_t s = (hipStream_t)stream;
     dim3 grid(M, tp_cdiv(D, 256)), grid_save(n_seq, tp_cdiv(D, 256));
-    if (dtype == TP_BF16) {
-        shift_mix_k<bf16_t><<<grid, 256, 0, s>>>((const bf16_t*)x, mu, state, slot_ids, cu_rows, row_seq, (bf16_t*)out, M, D, n_mix, one_row_each);
+    if (dtype == TP_BF16 && out_dtype == TP_BF16) {
+        shift_mix_k<bf16_t, bf16_t><<<grid, 256, 0, s>>>((const bf16_t*)x, mu, state, slot_ids, cu_rows, row_seq, (bf16_t*)out, M, D, n_mix, one_row_each);
         if (!one_row_each) shift_save_k<bf16_t><<<grid_save, 256, 0, s>>>((const bf16_t*)x, state, slot_ids, cu_rows, D);
-    } else if (dtype == TP_F32) {
-        shift_mix_k<float><<<grid, 256, 0, s>>>((const float*)x, mu, state, slot_ids, cu_rows, row_seq, (float*)out, M, D, n_mix, one_row_each);
+    } else if (dtype == TP_F32 && (out_dtype == TP_F32 || out_dtype == TP_BF16)) {
+        if (out_dtype == TP_F32) shift_mix_k<float, float><<<grid, 256, 0, s>>>((const float*)x, mu, state, slot_ids, cu_rows, row_seq, (float*)out, M, D, n_mix, one_row_each);
+        else shift_mix_k<float, bf16_t><<<grid, 256, 0, s>>>((const float*)x, mu, state, slot_ids, cu_rows, row_seq, (bf16_t*)out, M, D, n_mix, one_row_each);
         if (!one_row_each) shift_save_k<float><<<grid_save, 256, 0, s>>>((const float*)x, state, slot_ids, cu_rows, D);
-    } else return tp_fail("shift_mix: unknown dtype %d", dtype);
+    } else return tp_fail("shift_mix: no kernel from dtype %d to dtype %d", dtype, out_dtype);
     return tp_check_launch("shift_mix");
 }
 

@@ -102,11 +102,19 @@ class Model:
             out.append(states)
         return out
 
+    def entry_token_specs(self):
+        """For every schedule entry the paged tensors its mixer keeps by name beside its cache (none for a run on
+        another run's cache)."""
+        return [{} if e.cache_of is not None else
+                {"mixer." + name: spec for name, spec in self.layers[e.layer].block.mixer.token_specs().items()}
+                for e in self.schedule]
+
     def new_cache(self, max_tokens, max_context=None, max_slots=None, page_size=64):
         max_context = max_context or max_tokens
         max_slots = max_slots or max(1, -(-max_tokens // page_size))
         return ModelCache(self.entry_cache_specs(), max_tokens, max_context, max_slots, page_size,
-                          self.rt.dtype, self.rt.device, entry_states=self.entry_state_specs())
+                          self.rt.dtype, self.rt.device, entry_states=self.entry_state_specs(),
+                          entry_tokens=self.entry_token_specs())
 
     # --- the step -----------------------------------------------------------------------
     def step(self, cache, slots, tokens, counts=None, want=None):

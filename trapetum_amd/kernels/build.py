@@ -19,7 +19,7 @@ ARCH = "gfx950"
 FLAGS = ["--offload-arch=" + ARCH, "-O3", "-fPIC", "-std=c++17",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-result"]
 CORE_SOURCES = ["elementwise.hip", "gemm.hip", "gemm_skinny.hip", "gemm_mfma.hip", "gemv.hip", "gemm_rows8.hip", "attention_simple.hip", "sampling.hip", "probes.hip",
-                "conv.hip", "latent.hip", "moe.hip", "ssd.hip", "recurrent.hip"]
+                "conv.hip", "latent.hip", "moe.hip", "ssd.hip", "recurrent.hip", "attention_pooled.hip"]
 ATTN_SOURCES = ["attention_mfma.hip", "attention_prefill.hip"]      # decode steps; steps of many queries
 _NOISE = "is not a recognized feature for this target"
 

@@ -19,7 +19,7 @@ _CORE_SIGS = {
     "tp_add_rms_norm": [_P, _P, _I, _I, _L, _P, _F, _P, _F, _P, _I, _I, _I, _I, _P],
     "tp_scale_rows": [_P, _L, _F, _P],
     "tp_causal_conv": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
-    "tp_latent_prepare": [_P, _L, _I, _I, _I, _I, _I, _I, _P, _F, _P, _I, _P, _P, _P, _P, _I, _P, _I, _I, _P, _P, _I, _P],
+    "tp_latent_prepare": [_P, _L, _I, _I, _I, _I, _I, _I, _P, _F, _P, _I, _P, _P, _P, _P, _I, _P, _I, _I, _P, _P, _I, _P, _L, _P],
     "tp_head_linear": [_P, _L, _L, _P, _P, _L, _L, _I, _I, _I, _I, _I, _I, _P],
     "tp_route_top": [_P, _I, _I, _I, _I, _I, _P, _P, _P],
     "tp_expert_ffn_workspace_bytes": [_I, _I, _I, _I, _I, _I],
@@ -35,7 +35,14 @@ _CORE_SIGS = {
     "tp_kv_write": [_P, _L, _P, _L, _I, _I, _I, _I, _P, _P, _P, _P, _I, _P, _P, _I, _I, _P],
     "tp_gated_act": [_P, _P, _I, _I, _I, _I, _F, _F, _P],
     "tp_linear": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _F, _F, _P, _L, _I, _I, _P],
-    "tp_shift_mix": [_P, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
+    "tp_shift_mix": [_P, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P],
+    "tp_bias_act": [_P, _I, _P, _P, _I, _I, _I, _I, _P],
+    "tp_mul_sigmoid_heads": [_P, _L, _I, _P, _L, _I, _I, _I, _I, _P],
+    "tp_qkv_prepare": [_P, _L, _I, _P, _I, _I, _I, _I, _I, _P, _I, _I, _F, _P, _P, _P, _P, _I, _P],
+    "tp_pool_write": [_P, _L, _P, _L, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _I, _P, _P, _I, _P],
+    "tp_attn_pooled": [_P, _L, _P, _L, _P, _L, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _P, _I, _P, _P, _I,
+                       _F, _F, _I, _I, _P, _P],
+    "tp_talk_mix": [_P, _P, _P, _I, _I, _I, _I, _I, _P],
     "tp_unary_tanh": [_P, _I, _L, _P],
     "tp_weighted_sum": [_P, _F, _P, _F, _I, _P, _L, _P],
     "tp_head_norm_gate": [_P, _P, _P, _L, _I, _F, _P, _I, _I, _I, _I, _I, _P],
@@ -70,6 +77,7 @@ GATE_ACTIVATIONS = {"gelu_tanh": 0, "silu": 1, "relu": 2, "quick_gelu": 3}      
 HEAD_GATES = {"sigmoid": 0, "silu": 1}               # what `head_norm_gate` multiplies a normed head by: act(g)
 ROUTE_SCORES = {"softmax": 0, "sigmoid": 1}          # how a router's logits become scores
 CONV_ACTIVATIONS = {None: 0, "silu": 1}
+BIAS_ACTIVATIONS = {None: 0, "gelu_erf": 1}          # what `bias_act` applies after the bias
 GATE_GROUP = 16
 
 
@@ -299,15 +307,23 @@ class HipOps:
 
     # ---- attention through a cached latent ---------------------------------------------------------------------
     def latent_prepare(self, proj, H, dn, dr, R, gain, eps, inv_freq, rot, row_seq, row_pos, new_len, table, pool, rows_cap,
-                       own=True, out_dtype=None):
-        """proj [M, H (dr + dn) (+ dr + R)]: per head [rotated | unrotated] query parts, then (own) [key part | latent].
+                       own=True, out_dtype=None, tail=None, write=True):
+        """proj [M, H (dr + dn) (+ dr + R)]: per head [rotated | unrotated] query parts, then (own) [key part | latent];
+        tail: the [key part | latent] as rows of their own [M, dr + R] (then proj holds the queries only).  write False:
+        the step's rows are returned and not cached (the caller caches them after its attention has read the cache).
         Returns q [M, H (dr + R)] with every head's first dr elements set (the rotated query part; the rest is left
         for `head_linear`) and, when own, the step's rows [rope(key part) | rmsnorm(latent) * gain] [M, dr + R], which
         are also written into the cache pool [pages, 1, page, dr + R]."""
         self._dev(proj, gain, inv_freq, row_seq, row_pos, new_len, table, pool)
         m = proj.shape[0]
         stride = self._rows(proj, "latent_prepare proj")
-        width = H * (dr + dn) + ((dr + R) if own else 0)
+        width = H * (dr + dn) + ((dr + R) if own and tail is None else 0)
+        tail_stride = 0
+        if tail is not None:
+            self._dev(tail)
+            tail_stride = self._rows(tail, "latent_prepare tail")
+            if not own or tuple(tail.shape) != (m, dr + R) or tail.dtype != proj.dtype:
+                raise KernelError(f"latent_prepare: the key part and latent as rows of their own must be [{m}, {dr + R}] of {proj.dtype}")
         if proj.shape[1] != width or (out_dtype is not None and out_dtype != proj.dtype):
             raise KernelError(f"latent_prepare: rows of {proj.shape[1]} columns, this geometry needs {width} of the output's dtype")
         if rot and (inv_freq is None or inv_freq.dtype != torch.float32 or inv_freq.numel() != rot // 2):
@@ -326,9 +342,10 @@ class HipOps:
             mine = torch.empty((m, dr + R), dtype=proj.dtype, device=self.device)
         self._call(self.lib, "tp_latent_prepare", proj.data_ptr(), stride, _code(proj.dtype), m, H, dn, dr, R,
                    gain.data_ptr() if own else None, float(eps), inv_freq.data_ptr() if rot else None, int(rot),
-                   row_seq.data_ptr(), row_pos.data_ptr(), new_len.data_ptr(), table.data_ptr() if own else None, table_w,
-                   pool.data_ptr() if own else None, page, rows_cap if own else 0, q.data_ptr(),
-                   mine.data_ptr() if own else None, 1 if own else 0, self._stream())
+                   row_seq.data_ptr(), row_pos.data_ptr(), new_len.data_ptr(), table.data_ptr() if own and write else None, table_w,
+                   pool.data_ptr() if own and write else None, page, rows_cap if own and write else 0, q.data_ptr(),
+                   mine.data_ptr() if own else None, 1 if own else 0, tail.data_ptr() if tail is not None else None, tail_stride,
+                   self._stream())
         return q, mine
 
     def head_linear(self, x, w, out=None):
@@ -475,10 +492,10 @@ class HipOps:
                 raise KernelError(f"{what}: cu_rows, row_seq and slot_ids must be int32 of the step's geometry")
         return n_seq
 
-    def shift_mix(self, x, mu, state, slot_ids, cu_rows, row_seq, one_row_each=False):
+    def shift_mix(self, x, mu, state, slot_ids, cu_rows, row_seq, one_row_each=False, out_dtype=None):
         """out[s, r] = x[r] + (x[r - 1] - x[r]) * mu[s] within each sequence; the row before a sequence's first row of
         the step is state[slot] (float32 [slots, D]), which then takes the sequence's last row.  mu float32 [S, D];
-        returns [S, M, D] of x's dtype."""
+        returns [S, M, D] of x's dtype, or of out_dtype (float32 rows may give bfloat16 mixes)."""
         self._dev(x, mu, state, slot_ids, cu_rows, row_seq)
         if x.dim() != 2 or not x.is_contiguous():
             raise KernelError("shift_mix: rows must be a contiguous matrix")
@@ -488,9 +505,9 @@ class HipOps:
         if state.dtype != torch.float32 or state.dim() != 2 or state.shape[1] != d or not state.is_contiguous():
             raise KernelError(f"shift_mix: the state must be contiguous float32 [slots, {d}]")
         n_seq = self._geometry("shift_mix", m, slot_ids, cu_rows, row_seq)
-        out = torch.empty((mu.shape[0], m, d), dtype=x.dtype, device=self.device)
+        out = torch.empty((mu.shape[0], m, d), dtype=out_dtype or x.dtype, device=self.device)
         self._call(self.lib, "tp_shift_mix", x.data_ptr(), _code(x.dtype), mu.data_ptr(), mu.shape[0], state.data_ptr(), slot_ids.data_ptr(),
-                   cu_rows.data_ptr(), row_seq.data_ptr(), out.data_ptr(), m, n_seq, d, 1 if one_row_each else 0, self._stream())
+                   cu_rows.data_ptr(), row_seq.data_ptr(), out.data_ptr(), _code(out.dtype), m, n_seq, d, 1 if one_row_each else 0, self._stream())
         return out
 
     def unary_(self, x, name):
@@ -637,6 +654,32 @@ class HipOps:
         self._call(self.lib, "tp_mul_sigmoid", x.data_ptr(), xs, g.data_ptr(), gs, _code(x.dtype), x.shape[0], x.shape[1], self._stream())
         return x
 
+    def mul_sigmoid_heads(self, x, g, heads):
+        """x[r, h, :] *= sigmoid(g[r, h]), in place: x [M, heads * per] (a view of wider rows may do), g [M, heads]."""
+        self._dev(x, g)
+        xs, gs = self._rows(x, "mul_sigmoid_heads rows"), self._rows(g, "mul_sigmoid_heads gates")
+        if g.shape != (x.shape[0], heads) or x.shape[1] % heads:
+            raise KernelError(f"mul_sigmoid_heads: rows {tuple(x.shape)} and gates {tuple(g.shape)} do not fit {heads} heads")
+        self._call(self.lib, "tp_mul_sigmoid_heads", x.data_ptr(), xs, _code(x.dtype), g.data_ptr(), gs, _code(g.dtype), x.shape[0], heads,
+                   x.shape[1] // heads, self._stream())
+        return x
+
+    def bias_act(self, rows, bias, activation, out_dtype):
+        """act(rows + bias) in float32, rounded once to out_dtype: rows [M, N] float32 or bfloat16, bias float32 [N] or None;
+        activation: one of BIAS_ACTIVATIONS."""
+        if activation not in BIAS_ACTIVATIONS:
+            raise KernelError(f"bias_act: activation '{activation}' has no kernel ({', '.join(str(a) for a in BIAS_ACTIVATIONS)})")
+        self._dev(rows, bias)
+        if rows.dim() != 2 or not rows.is_contiguous():
+            raise KernelError("bias_act: rows must be a contiguous matrix")
+        m, n = rows.shape
+        if bias is not None and (bias.dtype != torch.float32 or bias.numel() != n or not bias.is_contiguous()):
+            raise KernelError(f"bias_act: the bias must be contiguous float32 [{n}]")
+        out = torch.empty((m, n), dtype=out_dtype, device=self.device)
+        self._call(self.lib, "tp_bias_act", rows.data_ptr(), _code(rows.dtype), bias.data_ptr() if bias is not None else None, out.data_ptr(),
+                   _code(out_dtype), m, n, BIAS_ACTIVATIONS[activation], self._stream())
+        return out
+
     MAX_SLICED_WIDTH = 8192        # widest row `add_rms_norm` takes in K slices
 
     def rows(self, rows, dtype):
@@ -712,6 +755,103 @@ class HipOps:
         self._call(self.lib, "tp_kv_write", k.data_ptr(), ks, v.data_ptr(), vs, _code(k.dtype), m, KV, hd, row_seq.data_ptr(),
                    row_pos.data_ptr(), new_len.data_ptr(), table.data_ptr(), table.shape[1], k_pool.data_ptr(),
                    v_pool.data_ptr(), k_pool.shape[2], rows_cap, self._stream())
+
+    # ---- attention over a window and pooled blocks ------------------------------------------------------
+    def qkv_prepare(self, x, bias, H, KV, row, dim, inv_freq, rotary_dim, row_pos, unit_eps, out_dtype, pairing="halves"):
+        """A step's projected rows [M, (H + 2 KV) row] (or [M, H row] with KV = 0), float32 or out_dtype: bias, rotation of
+        every query and key head's first rotary_dim elements by its row's position, then (unit_eps not None) every
+        query and key head over the root mean square of its `dim` elements; everything in float32, rounded once.
+        Returns q [M, H row], k, v [M, KV row] (None with KV = 0) of out_dtype."""
+        self._dev(x, bias, inv_freq, row_pos)
+        xs = self._rows(x, "qkv_prepare rows")
+        m = x.shape[0]
+        if x.shape[1] != (H + 2 * KV) * row:
+            raise KernelError(f"qkv_prepare: rows of {x.shape[1]} columns, {H} + 2 x {KV} heads of {row} need {(H + 2 * KV) * row}")
+        if bias is not None and (bias.dtype != torch.float32 or bias.numel() != x.shape[1] or not bias.is_contiguous()):
+            raise KernelError(f"qkv_prepare: the bias must be contiguous float32 [{x.shape[1]}]")
+        if rotary_dim and (inv_freq is None or inv_freq.dtype != torch.float32 or inv_freq.numel() != rotary_dim // 2):
+            raise KernelError(f"qkv_prepare: a rotation over {rotary_dim} needs float32 inv_freq [{rotary_dim // 2}]")
+        if row_pos.dtype != torch.int32 or row_pos.numel() != m:
+            raise KernelError("qkv_prepare: row_pos must be int32, one entry per row")
+        if pairing not in ROPE_PAIRINGS:
+            raise KernelError(f"qkv_prepare: pairing '{pairing}' has no kernel")
+        q = torch.empty((m, H * row), dtype=out_dtype, device=self.device)
+        k = torch.empty((m, KV * row), dtype=out_dtype, device=self.device) if KV else None
+        v = torch.empty((m, KV * row), dtype=out_dtype, device=self.device) if KV else None
+        self._call(self.lib, "tp_qkv_prepare", x.data_ptr(), xs, _code(x.dtype), bias.data_ptr() if bias is not None else None, m, H, KV, row, dim,
+                   inv_freq.data_ptr() if rotary_dim else None, rotary_dim, ROPE_PAIRINGS[pairing],
+                   -1.0 if unit_eps is None else float(unit_eps), row_pos.data_ptr(), q.data_ptr(),
+                   k.data_ptr() if KV else None, v.data_ptr() if KV else None, _code(out_dtype), self._stream())
+        return q, k, v
+
+    def pool_write(self, k, v, KV, row, block, cu_rows, max_count, new_len, slot_ids, sums, table, k_blocks, v_blocks):
+        """The mean key and value of every block of `block` positions that the step completes, into the pools
+        [pages, KV, page, row] that keep one row per block (found through `table`); sums float32 [slots, 2, KV row]
+        carries an unfinished block's sums from step to step."""
+        self._dev(k, v, cu_rows, new_len, slot_ids, sums, table, k_blocks, v_blocks)
+        ks, vs = self._rows(k, "pool_write k"), self._rows(v, "pool_write v")
+        n = new_len.numel()
+        if k.shape != v.shape or k.shape[1] != KV * row or k.dtype != v.dtype:
+            raise KernelError("pool_write: k and v must be [rows, kv_heads * row] of one dtype")
+        for t, cnt in ((cu_rows, n + 1), (new_len, n), (slot_ids, n)):
+            if t.dtype != torch.int32 or t.numel() != cnt:
+                raise KernelError("pool_write: cu_rows, new_len and slot_ids must be int32 of the step's geometry")
+        if sums.dtype != torch.float32 or sums.dim() != 3 or tuple(sums.shape[1:]) != (2, KV * row) or not sums.is_contiguous():
+            raise KernelError(f"pool_write: the sums must be contiguous float32 [slots, 2, {KV * row}]")
+        for pool in (k_blocks, v_blocks):
+            if pool.dim() != 4 or pool.shape[1] != KV or pool.shape[3] != row or pool.dtype != k.dtype or not pool.is_contiguous():
+                raise KernelError(f"pool_write: a pool must be contiguous [pages, {KV}, page, {row}] of {k.dtype}")
+        if table.dtype != torch.int32 or table.dim() != 2 or table.shape[0] != n or table.stride(1) != 1 or table.stride(0) != table.shape[1]:
+            raise KernelError("pool_write: the page table must be contiguous int32 [sequences, pages]")
+        self._call(self.lib, "tp_pool_write", k.data_ptr(), ks, v.data_ptr(), vs, _code(k.dtype), n, int(max_count), KV, row, int(block),
+                   cu_rows.data_ptr(), new_len.data_ptr(), slot_ids.data_ptr(), sums.data_ptr(), table.data_ptr(), table.shape[1],
+                   k_blocks.data_ptr(), v_blocks.data_ptr(), k_blocks.shape[2], self._stream())
+
+    def attention_pooled(self, q, k, v, H, KV, hd, cu_rows, row_seq, row_pos, new_len, table, k_pool, v_pool, rows_cap,
+                         scale, softcap, window, blocks=None, all_values=False):
+        """Attention of the step's queries over the positions their window still holds (those before the step read in
+        place from the cache, the step's own rows from k and v) and, with blocks = (block size, page table, key pool,
+        value pool), over one pooled key and value per block of positions that lies wholly before the window; one
+        softmax over both.  Returns float32 [M, H, KV if all_values else 1, hd]: with all_values every query head's
+        weights are applied to the values of every kv head (what a mix of the heads' weights needs)."""
+        self._dev(q, k, v, cu_rows, row_seq, row_pos, new_len, table, k_pool, v_pool)
+        m = q.shape[0]
+        qs, ks, vs = self._rows(q, "attention_pooled q"), self._rows(k, "attention_pooled k"), self._rows(v, "attention_pooled v")
+        if q.shape[1] != H * hd or k.shape != (m, KV * hd) or v.shape != (m, KV * hd) or k.dtype != q.dtype or v.dtype != q.dtype:
+            raise KernelError(f"attention_pooled: q [rows, {H * hd}], k and v [rows, {KV * hd}] of one dtype, found {tuple(q.shape)}, {tuple(k.shape)}, {tuple(v.shape)}")
+        n = new_len.numel()
+        for t, cnt in ((cu_rows, n + 1), (row_seq, m), (row_pos, m)):
+            if t.dtype != torch.int32 or t.numel() != cnt:
+                raise KernelError("attention_pooled: cu_rows, row_seq and row_pos must be int32 of the step's geometry")
+        self._check_pools("attention_pooled", q.dtype, n, KV, hd, new_len, table, k_pool, v_pool)
+        page = k_pool.shape[2]
+        if blocks is not None:
+            block, btable, kb, vb = blocks
+            self._dev(btable, kb, vb)
+            self._check_pools("attention_pooled (blocks)", q.dtype, n, KV, hd, new_len, btable, kb, vb)
+            if kb.shape[2] != page or not window:
+                raise KernelError("attention_pooled: the blocks' pools have the cache's page size, and blocks need a window")
+        self_out = torch.empty((m, H, KV if all_values else 1, hd), dtype=torch.float32, device=self.device)
+        self._call(self.lib, "tp_attn_pooled", q.data_ptr(), qs, k.data_ptr(), ks, v.data_ptr(), vs, _code(q.dtype), m, H, KV, hd,
+                   cu_rows.data_ptr(), row_seq.data_ptr(), row_pos.data_ptr(), new_len.data_ptr(), table.data_ptr(), table.shape[1],
+                   k_pool.data_ptr(), v_pool.data_ptr(), page, rows_cap or 0,
+                   btable.data_ptr() if blocks else None, btable.shape[1] if blocks else 0, kb.data_ptr() if blocks else None,
+                   vb.data_ptr() if blocks else None, int(block) if blocks else 0,
+                   float(scale), float(softcap or 0.0), int(window or 0), 1 if all_values else 0, self_out.data_ptr(), self._stream())
+        return self_out
+
+    def talk_mix(self, a, talk, out_dtype):
+        """out[r, h] = sum_g talk[h, g] a[r, g, kv(h)]: a float32 [M, H, KV, hd] as `attention_pooled(all_values=True)`
+        gives it, talk float32 [H, H]; returns [M, H * hd] of out_dtype."""
+        self._dev(a, talk)
+        if a.dtype != torch.float32 or a.dim() != 4 or not a.is_contiguous():
+            raise KernelError("talk_mix: the heads' outputs must be contiguous float32 [rows, heads, kv heads, head_dim]")
+        m, H, KV, hd = a.shape
+        if talk.dtype != torch.float32 or tuple(talk.shape) != (H, H) or not talk.is_contiguous():
+            raise KernelError(f"talk_mix: the mixing matrix must be contiguous float32 [{H}, {H}]")
+        out = torch.empty((m, H * hd), dtype=out_dtype, device=self.device)
+        self._call(self.lib, "tp_talk_mix", a.data_ptr(), talk.data_ptr(), out.data_ptr(), _code(out_dtype), m, H, KV, hd, self._stream())
+        return out
 
     # ---- matrix products -----------------------------------------------------------------------------
     def _linear(self, x, w, out_dtype, epilogue, cap, units, defer=False, act=0, out=None, limit=float("inf"), shift=0.0):

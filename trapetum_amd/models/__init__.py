@@ -1,2 +1,2 @@
 """Architectures; importing this package registers the built-in ones."""
-from . import besulix, gemma2, golepel, lutovik   # noqa: F401
+from . import besulix, gemma2, golepel, lutovik, vogunex   # noqa: F401

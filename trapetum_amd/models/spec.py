@@ -15,7 +15,7 @@ PartRef = Tuple[str, dict]          # (registered name, constructor parameters)
 class TensorSpec:
     """One tensor a part needs: its shape and how a random model fills it."""
     shape: tuple
-    init: str = "matrix"            # "matrix", "norm", "embedding": which sigma; "gain": one plus "norm"; "zeros"; "ones"
+    init: str = "matrix"            # "matrix", "norm", "embedding": which sigma; "gain": one plus "norm"; "talk": unit matrix plus noise; "zeros"; "ones"
     dtype: str = "float"            # "float": kept as stored (bf16, or fp32 if stored so); "int": int32 table
     free: tuple = ()                # dimensions whose size the checkpoint gives (no configuration key names it): `shape` there
                                     # holds what a random model takes, and the part reads the real size when it binds

@@ -31,6 +31,18 @@ back by -p, so that the weighted sum is read in the query's frame.  Chunks, temp
 every attention kernel (a chunk is a window whose start does not move with the query; the sink is added to the sum
 when a query's keys are done, in the kernel that normalises); the values' two rotations are launches of the rotation
 kernel.  A decode step of such a layer is not the one fused launch: its projections carry biases and its values turn.
+
+A third family of parameters makes the layer an attention over a window plus pooled blocks whose heads talk:
+`unit_norm_eps` (every query and key head is divided by its root mean square after the rotation: a norm without a
+gain), `pool` P (beside the `window` W positions back a query at p sees one key and value for every block of P
+positions b P .. b P + P - 1 with b P + P - 1 <= p - W, the mean of the block's cached keys and of its values; the
+positions between the last such block and the window are not seen at all) and `talk` (a matrix [heads, heads] that
+mixes the heads' softmax weights, w_h <- sum_g T[h, g] w_g, before head h applies them to the values of its own kv
+head).  Any of the three takes the layer to `ops.qkv_prepare` (bias, rotation and unit norm in float32 from the
+product's float32 sums, one rounding), `ops.pool_write` (the block means go to a paged pool of their own that keeps
+one row per P tokens; an unfinished block's sums wait in a float32 state), `ops.attention_pooled` and
+`ops.talk_mix`.  The cache's ring keeps the window only; the step's rows are cached after the attention in every
+kind of step, so one sequence of launches serves prompts, portions of prompts and decode steps.
 """
 from ..cache.store import TokenSpec
 from ..models.spec import TensorSpec
@@ -43,7 +55,8 @@ class Attention(Mixer):
                  softcap=None, window=None, position=("none", {}), value_dim=None, output_gate=False, own_kv=True,
                  precise_weights=False,
                  tensors=("q_proj.weight", "k_proj.weight", "v_proj.weight", "o_proj.weight", "g_proj.weight"),
-                 bias_suffix=None, chunk=None, head_temperature=None, sink=None, value_rotation=None):
+                 bias_suffix=None, chunk=None, head_temperature=None, sink=None, value_rotation=None,
+                 unit_norm_eps=None, pool=None, talk=None):
         """value_dim: elements of a value head when they differ from a key's head_dim.  output_gate: the heads' outputs
         are multiplied by sigmoid(W_g x) before the output projection.  own_kv False: the layer has no key and value
         projections; its schedule entry names the run whose cache it reads.  precise_weights: the softmax weights meet
@@ -51,7 +64,9 @@ class Attention(Mixer):
         otherwise; a decode step's are float32 anyway).  tensors: local names of W_q, W_k, W_v, W_o (and W_g).
         bias_suffix: q, k and v have biases, named like their matrices with this suffix.  chunk: positions per chunk.
         head_temperature, sink: local names of float vectors [heads].  value_rotation: the base theta of the values'
-        rotation by their position."""
+        rotation by their position.  unit_norm_eps: the eps of the norm without gain on every query and key head (None:
+        no such norm).  pool: positions per pooled block before the window.  talk: local name of the matrix
+        [heads, heads] that mixes the heads' softmax weights."""
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads are no multiple of {num_kv_heads} kv heads")
         self.hidden_size = hidden_size
@@ -83,6 +98,15 @@ class Attention(Mixer):
         self.per_head = bool(self.chunk or head_temperature or sink)
         if (self.per_head or value_rotation is not None) and (self.output_gate or not self.own_kv):
             raise ValueError("chunks, temperatures, sinks and rotated values go with an ungated attention on its own cache")
+        self.unit_norm_eps = None if unit_norm_eps is None else float(unit_norm_eps)
+        self.pool = int(pool) if pool else 0
+        self.talk_name = talk
+        self.pooled = self.unit_norm_eps is not None or bool(self.pool) or talk is not None
+        if self.pooled and (self.per_head or value_rotation is not None or not self.own_kv):
+            raise ValueError("unit norms, pooled blocks and talking heads go with an attention on its own cache, without chunks, "
+                             "temperatures, sinks or rotated values")
+        if self.pool and not self.window:
+            raise ValueError("pooled blocks stand before a window: the layer needs one")
 
     @property
     def reach(self):
@@ -105,11 +129,27 @@ class Attention(Mixer):
             specs[self.temperature_name] = TensorSpec((self.num_heads,), init="gain")
         if self.sink_name:
             specs[self.sink_name] = TensorSpec((self.num_heads,), init="norm")
+        if self.talk_name:
+            specs[self.talk_name] = TensorSpec((self.num_heads, self.num_heads), init="talk")
         return specs
 
     def cache_spec(self):
         per_token = (self.num_kv_heads, self.row)
         return TokenSpec.of(self.reach or None, k=per_token, v=per_token)
+
+    def token_specs(self):
+        """The pooled blocks: one mean key and value per `pool` tokens, of all tokens."""
+        if not self.pool:
+            return {}
+        per_block = (self.num_kv_heads, self.row)
+        return {"blocks": TokenSpec.of(None, every=self.pool, k=per_block, v=per_block)}
+
+    def state_specs(self):
+        """The sums of the keys and of the values of the block that is not finished yet."""
+        if not self.pool:
+            return {}
+        from ..cache.store import StateSpec
+        return {"block_sums": StateSpec((2, self.num_kv_heads * self.row), "float32")}
 
     def _heads(self, w, heads, size, turned=False):
         """[heads * size, d] -> [heads * row, d]: zero rows fill a head up to `row`.  turned: a rotation of neighbouring
@@ -148,6 +188,9 @@ class Attention(Mixer):
                                     for s, heads, size, t in sides]).float().contiguous()
         self.temperature = tensors[self.temperature_name].float().contiguous() if self.temperature_name else None
         self.sink = tensors[self.sink_name].float().contiguous() if self.sink_name else None
+        self.talk = None
+        if self.pooled:            # heads that do not talk are mixed by the unit matrix, in the same launch that rounds
+            self.talk = (tensors[self.talk_name].float() if self.talk_name else torch.eye(H, device=self.w_o.device)).contiguous()
         self.value_freq = self.value_back = None
         if self.value_position is not None:
             self.value_freq = self.value_position.inv_freq(rt.device)
@@ -165,7 +208,40 @@ class Attention(Mixer):
         ctx.ops.rope_kv_write(rows, None, None, heads, 0, self.row, freq, self.value_dim, ctx.row_seq, ctx.row_pos, ctx.new_len,
                               None, None, None, 0, write=False)
 
+    def _forward_pooled(self, ctx, x, site):
+        import torch
+        ops = ctx.ops
+        H, KV, hd = self.num_heads, self.num_kv_heads, self.row
+        if ctx.cache_owner != ctx.entry:
+            raise ValueError("an attention with unit norms, pooled blocks or talking heads runs on its own cache")
+        if site.spec.window is not None and not 0 < self.reach <= site.spec.window:
+            raise ValueError(f"this attention sees {self.reach or 'all'} keys back, the cache it reads keeps {site.spec.window}")
+        table = ctx.page_table(site.group_index)
+        k_pool, v_pool = site.tensor("k"), site.tensor("v")
+        rows_cap = site.rows_cap or 0
+        qkv = ops.linear(x, self.w_qkv, torch.float32)                # float32 sums: bias, rotation and norm before any rounding
+        q, k, v = ops.qkv_prepare(qkv, self.b_qkv, H, KV, hd, self.head_dim, self.inv_freq, self.position.rotary_dim, ctx.row_pos,
+                                  self.unit_norm_eps, ctx.dtype)
+        blocks = None
+        if self.pool:
+            bsite = self.tokens(ctx, "blocks")
+            btable = ctx.page_table(bsite.group_index)
+            kb, vb = bsite.tensor("k"), bsite.tensor("v")
+            # the blocks this step completes are seen by its own later queries: their means are written first (the
+            # pool keeps every block, so nothing a query still needs is overwritten)
+            ops.pool_write(k, v, KV, hd, self.pool, ctx.cu_rows, ctx.max_count, ctx.new_len, ctx.slot_ids,
+                           self.state(ctx, "block_sums"), btable, kb, vb)
+            blocks = (self.pool, btable, kb, vb)
+        a = ops.attention_pooled(q, k, v, H, KV, hd, ctx.cu_rows, ctx.row_seq, ctx.row_pos, ctx.new_len, table, k_pool, v_pool,
+                                 rows_cap, self.query_scale, self.softcap, self.window, blocks=blocks,
+                                 all_values=self.talk_name is not None)
+        out = ops.talk_mix(a, self.talk, ctx.dtype)
+        ops.kv_write(k, v, KV, hd, ctx.row_seq, ctx.row_pos, ctx.new_len, table, k_pool, v_pool, rows_cap)
+        return self._project_out(ctx, x, out)
+
     def forward(self, ctx, x, site):
+        if self.pooled:
+            return self._forward_pooled(ctx, x, site)
         ops = ctx.ops
         H, KV, hd = self.num_heads, self.num_kv_heads, self.row
         Q, KVD = H * hd, KV * hd

@@ -67,6 +67,15 @@ class Mixer(Part):
         token and states, or several states)."""
         return {}
 
+    def token_specs(self):
+        """{name: TokenSpec} of further paged tensors the mixer keeps by name (`self.tokens(ctx, name)`): rows at
+        another rate than its cache_spec's, one per block of `every` tokens."""
+        return {}
+
+    def tokens(self, ctx, name):
+        """The site of the running entry's paged tensors `name`: `.tensor(n)`, `.group_index` for `ctx.page_table`."""
+        return ctx.cache.entry_site(ctx.entry, "mixer." + self.state_scope + name)
+
     def state(self, ctx, name):
         """The running entry's state `name` of this mixer: [slots + 1, *shape]."""
         return ctx.cache.entry_state(ctx.entry, "mixer." + self.state_scope + name)

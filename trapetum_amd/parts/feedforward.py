@@ -46,4 +46,35 @@ class GatedMLP(FeedForward):
         return ctx.ops.linear(act, self.w_down, ctx.dtype, defer=True)
 
 
+class BiasedMLP(FeedForward):
+    """down(act(up x + b_up)) + b_down: one product up, one down, both with a bias, no gate.  The first product's
+    float32 sums take the bias and the activation before they are rounded; the second leaves float32 rows for the
+    residual add."""
+
+    def __init__(self, hidden_size, intermediate_size, activation="gelu_erf", tensors=("up", "down"), bias_suffix=".b"):
+        """activation: gelu_erf, the exact x Phi(x).  tensors: local names of the two matrices; a bias is named like its
+        matrix with bias_suffix."""
+        self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
+        self.activation = activation
+        self.names = tuple(tensors)
+        self.bias_suffix = bias_suffix
+
+    def tensor_specs(self):
+        d, i, (up, dn), b = self.hidden_size, self.intermediate_size, self.names, self.bias_suffix
+        return {up: TensorSpec((i, d)), up + b: TensorSpec((i,), init="norm"),
+                dn: TensorSpec((d, i)), dn + b: TensorSpec((d,), init="norm")}
+
+    def bind(self, tensors, rt):
+        self.rt = rt
+        (up, dn), b = self.names, self.bias_suffix
+        self.w_up, self.w_down = rt.matrix(tensors[up]), rt.matrix(tensors[dn])
+        self.b_up, self.b_down = tensors[up + b].float().contiguous(), tensors[dn + b].float().contiguous()
+
+    def forward(self, ctx, x, out=None):
+        import torch
+        act = ctx.ops.bias_act(ctx.ops.linear(x, self.w_up, torch.float32), self.b_up, self.activation, ctx.dtype)
+        return ctx.ops.linear(act, self.w_down, torch.float32, bias=self.b_down)
+
+
 register_part("feed_forward", "gated_mlp", GatedMLP)
+register_part("feed_forward", "biased_mlp", BiasedMLP)

@@ -12,6 +12,12 @@ attention uses (its `k` and `v` pools are one tensor here); the rotated part sta
 kernels rotate a head's leading elements.  A step's cost is then one read of rope_dim + rank elements per cached
 token for all heads, instead of heads * (dim + vdim).
 
+Further parameters: `query_rank` (the queries go through a latent of their own, q = W_uq rmsnorm(W_dq h) * w_qnorm,
+instead of one product), `window` W (the query at p sees the positions p - W + 1 .. p; the cache then keeps a ring),
+`output_gate` (head h's output is multiplied by sigmoid(W_g h)_h, one number per head and token) and a rotation of
+neighbouring pairs (2f, 2f + 1), carried out as the rotation of halves on projection rows reordered at bind (queries
+and key part alike: every score is the same sum in another order).
+
 A run with `own_latent=False` has no W_dkv: it attends over what the run named by its schedule entry's `cache_of`
 cached (and, in the step that caches them, over that run's rows of this step), with its own queries, W_uk, W_uv, W_o.
 """
@@ -26,7 +32,12 @@ class LatentAttention(Mixer):
 
     def __init__(self, hidden_size, num_heads, nope_dim, rope_dim, value_dim, latent_rank, scale, latent_eps,
                  position=("none", {}), own_latent=True,
-                 tensors=("q", "dkv", "dkv.norm", "uk", "uv", "o")):
+                 tensors=("q", "dkv", "dkv.norm", "uk", "uv", "o"), query_rank=None, query_tensors=("dq", "dq.norm", "uq"),
+                 window=None, output_gate=None, precise_weights=False):
+        """query_rank: size of the queries' latent (None: queries are one product, tensor `q`); query_tensors: local
+        names of W_dq, the latent's gain and W_uq.  window: positions back a query sees, its own included (None: all).
+        output_gate: local name of W_g [heads, hidden] (None: no gate).  precise_weights: softmax weights of 16 bits of
+        mantissa in the matrix-core kernel of many queries."""
         self.hidden_size, self.num_heads = int(hidden_size), int(num_heads)
         self.nope_dim, self.rope_dim, self.value_dim, self.rank = int(nope_dim), int(rope_dim), int(value_dim), int(latent_rank)
         self.scale = float(scale)
@@ -35,9 +46,12 @@ class LatentAttention(Mixer):
         self.position = build_part("position", position)
         if self.position.rotary_dim > self.rope_dim:
             raise ValueError(f"rotary_dim {self.position.rotary_dim} exceeds the rotated part of {self.rope_dim}")
-        if self.position.rotary_dim and self.position.pairing != "halves":
-            raise ValueError("the latent's rotation pairs halves; no kernel turns neighbours here")
         self.names = dict(zip(("q", "dkv", "dkv_norm", "uk", "uv", "o"), tensors))
+        self.query_rank = int(query_rank) if query_rank else 0
+        self.names.update(zip(("dq", "dq_norm", "uq"), query_tensors))
+        self.window = int(window) if window else 0
+        self.gate_name = output_gate
+        self.precise_weights = bool(precise_weights)
 
     @property
     def row(self):
@@ -46,16 +60,23 @@ class LatentAttention(Mixer):
 
     def tensor_specs(self):
         n, d, H = self.names, self.hidden_size, self.num_heads
-        specs = {n["q"]: TensorSpec((H * (self.nope_dim + self.rope_dim), d)),
-                 n["uk"]: TensorSpec((H * self.nope_dim, self.rank)), n["uv"]: TensorSpec((H * self.value_dim, self.rank)),
-                 n["o"]: TensorSpec((d, H * self.value_dim))}
+        qd = H * (self.nope_dim + self.rope_dim)
+        if self.query_rank:
+            specs = {n["dq"]: TensorSpec((self.query_rank, d)), n["dq_norm"]: TensorSpec((self.query_rank,), init="gain"),
+                     n["uq"]: TensorSpec((qd, self.query_rank))}
+        else:
+            specs = {n["q"]: TensorSpec((qd, d))}
+        if self.gate_name:
+            specs[self.gate_name] = TensorSpec((H, d))
+        specs.update({n["uk"]: TensorSpec((H * self.nope_dim, self.rank)), n["uv"]: TensorSpec((H * self.value_dim, self.rank)),
+                 n["o"]: TensorSpec((d, H * self.value_dim))})
         if self.own_latent:
             specs[n["dkv"]] = TensorSpec((self.rank + self.rope_dim, d))
             specs[n["dkv_norm"]] = TensorSpec((self.rank,), init="gain")
         return specs
 
     def cache_spec(self):
-        return TokenSpec.of(None, latent=(1, self.row))
+        return TokenSpec.of(self.window or None, latent=(1, self.row))
 
     def bind(self, tensors, rt):
         import torch
@@ -63,15 +84,25 @@ class LatentAttention(Mixer):
         n, H, dn, dr, dv, R = self.names, self.num_heads, self.nope_dim, self.rope_dim, self.value_dim, self.rank
         # queries head by head as [rotated | unrotated], the down-projection as [rotated key part | latent]: the order
         # of a cached row, and of the query that meets it
-        wq = tensors[n["q"]].reshape(H, dn + dr, -1)
-        wq = torch.cat([wq[:, dn:], wq[:, :dn]], dim=1).reshape(H * (dn + dr), -1)
-        if self.own_latent:
-            wd = tensors[n["dkv"]]
-            self.w_in = rt.matrix(torch.cat([wq, wd[R:], wd[:R]], dim=0).contiguous())
-            self.latent_gain = tensors[n["dkv_norm"]].float().contiguous()
+        rot = self.position.rotary_dim
+        turned = list(range(dr))                         # the rotated part's rows in the order the kernels turn them
+        if rot and self.position.pairing == "neighbours":
+            turned = list(range(0, rot, 2)) + list(range(1, rot, 2)) + list(range(rot, dr))
+        wq = tensors[n["uq"] if self.query_rank else n["q"]].reshape(H, dn + dr, -1)
+        wq = torch.cat([wq[:, dn:][:, turned], wq[:, :dn]], dim=1).reshape(H * (dn + dr), -1)
+        wd = tensors[n["dkv"]] if self.own_latent else None
+        tail = torch.cat([wd[R:][turned], wd[:R]], dim=0) if self.own_latent else None
+        self.latent_gain = tensors[n["dkv_norm"]].float().contiguous() if self.own_latent else None
+        self.w_in = self.w_tail = self.w_dq = self.w_uq = self.query_gain = None
+        if self.query_rank:
+            self.w_dq = rt.matrix(tensors[n["dq"]].contiguous())
+            self.query_gain = tensors[n["dq_norm"]].float().contiguous()
+            self.w_uq = rt.matrix(wq.contiguous())
+            if self.own_latent:
+                self.w_tail = rt.matrix(tail.contiguous())
         else:
-            self.w_in = rt.matrix(wq.contiguous())
-            self.latent_gain = None
+            self.w_in = rt.matrix((torch.cat([wq, tail], dim=0) if self.own_latent else wq).contiguous())
+        self.w_gate = rt.matrix(tensors[self.gate_name].contiguous()) if self.gate_name else None
         self.w_absorb = rt.matrix(tensors[n["uk"]].reshape(H, dn, R).transpose(1, 2).contiguous())     # [H, rank, dim]
         self.w_up = rt.matrix(tensors[n["uv"]].reshape(H, dv, R).contiguous())                         # [H, vdim, rank]
         self.w_o = rt.matrix(tensors[n["o"]])
@@ -89,12 +120,23 @@ class LatentAttention(Mixer):
         pool = site.tensor("latent")                              # [pages, 1, page, rope_dim + rank]
         rows_cap = site.rows_cap or 0
         m = x.shape[0]
-        proj = ops.linear(x, self.w_in, ctx.dtype)                # [M, H (dr + dn) (+ dr + rank)]
+        import torch
+        tail = None
+        if self.query_rank:
+            cq = ops.rms_norm(ops.linear(x, self.w_dq, torch.float32), self.query_gain, self.latent_eps, ctx.dtype)
+            proj = ops.linear(cq, self.w_uq, ctx.dtype)           # [M, H (dr + dn)]
+            if owns:
+                tail = ops.linear(x, self.w_tail, ctx.dtype)      # [M, dr + rank]
+        else:
+            proj = ops.linear(x, self.w_in, ctx.dtype)            # [M, H (dr + dn) (+ dr + rank)]
+        # A step that continues sequences by several tokens reads the ring as earlier steps left it, so its rows are
+        # cached after the attention: in a ring they may take the places of positions that its first queries still see.
+        late = owns and ctx.mode == "extend" and bool(rows_cap)
         # rotations, the latent's norm and the cache write in one launch: the queries' rotated parts go to their
         # places in q, the step's rows [r | c] to `mine` and into the cache
         q, mine = ops.latent_prepare(proj, H, dn, dr, R, self.latent_gain, self.latent_eps, self.inv_freq,
                                      self.position.rotary_dim, ctx.row_seq, ctx.row_pos, ctx.new_len, table, pool,
-                                     rows_cap, own=owns, out_dtype=ctx.dtype)
+                                     rows_cap, own=owns, out_dtype=ctx.dtype, tail=tail, write=not late)
         ops.head_linear(proj[:, :H * (dr + dn)].view(m, H, dr + dn)[:, :, dr:], self.w_absorb, q.view(m, H, row)[:, :, dr:])
         if ctx.mode == "decode":
             # All heads share the one kv head.  A block of the decode kernel forms the weighted sums of a kv head's
@@ -105,7 +147,7 @@ class LatentAttention(Mixer):
             # 552 keys 46.8 / 35.5 / 30.0 / 36.5.
             keys = ctx.max_rows_visible(site)
             per = next(g for g in (self.DECODE_GROUP_LONG if keys >= self.LONG_KEYS else self.DECODE_GROUP, 4, 2, 1) if H % g == 0)
-            out = ops.attention_decode(q, H, 1, row, ctx.new_len, table, pool, pool, rows_cap, self.scale, 0.0, 0,
+            out = ops.attention_decode(q, H, 1, row, ctx.new_len, table, pool, pool, rows_cap, self.scale, 0.0, self.window,
                                        ctx.dtype, max_keys=keys, head_groups=H // per,
                                        splits=ops.decode_splits(m * (H // per), 1, row, keys))
         else:
@@ -114,10 +156,16 @@ class LatentAttention(Mixer):
             else:
                 mine = ctx.step_rows_of(ctx.cache_owner)["latent"]
             extend = ctx.mode == "extend"
-            out = ops.attention_prefill(q, mine, mine, H, 1, row, ctx.cu_rows, ctx.max_count, self.scale, 0.0, 0, ctx.dtype,
+            out = ops.attention_prefill(q, mine, mine, H, 1, row, ctx.cu_rows, ctx.max_count, self.scale, 0.0, self.window, ctx.dtype,
                                         row_seq=ctx.row_seq, row_pos=ctx.row_pos,
-                                        cached=(ctx.new_len, table, pool, pool, rows_cap) if extend else None)
+                                        cached=(ctx.new_len, table, pool, pool, rows_cap) if extend else None,
+                                        wide_weights=self.precise_weights)
+            if late:
+                row_seq, row_pos, new_len = ctx.row_seq, ctx.row_pos, ctx.new_len
+                ctx.after_readers(lambda: ops.kv_write(mine, mine, 1, row, row_seq, row_pos, new_len, table, pool, pool, rows_cap))
         heads = ops.head_linear(out.view(m, H, row)[:, :, dr:], self.w_up, None)      # [M, H, vdim]
+        if self.w_gate is not None:
+            ops.mul_sigmoid_heads(heads.view(m, H * dv), ops.linear(x, self.w_gate, torch.float32), H)
         return ops.linear(heads.view(m, H * dv), self.w_o, ctx.dtype, defer=True)
 
 

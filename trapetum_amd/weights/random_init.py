@@ -53,6 +53,9 @@ class RandomWeights:
             return torch.zeros(ts.shape, dtype=self.store_dtype)
         if ts.init == "ones":
             return torch.ones(ts.shape, dtype=self.store_dtype)
+        if ts.init == "talk":                                 # a square mixing matrix: the unit matrix plus noise
+            noise = torch.empty(ts.shape, dtype=torch.float32).normal_(0.0, 1.0, generator=g) * 0.25
+            return (torch.eye(ts.shape[0]) + noise).to(self.store_dtype)
         sigma = self.sigma_norm if ts.init in ("norm", "gain") else self.sigma
         shift = 1.0 if ts.init == "gain" else 0.0          # a gain that is used as stored lies around one
         if self.draw_on is not None:
