@@ -3,11 +3,11 @@ prompt then decoding, portions, unequal batches on reused slots and pages, sharp
 (model, cfg, plain config, plain weights, tolerance); the plain implementation is chosen by the design's name."""
 import torch
 
-from .plain import besulix_plain, golepel_plain, lutovik_plain
+from .plain import besulix_plain, golepel_plain, lutovik_plain, vogunex_plain
 from .tiny import random_tokens, rel_l2
 from . import trace_schedules as ts
 
-PLAIN = {"Besulix": besulix_plain, "Golepel": golepel_plain, "Lutovik": lutovik_plain}
+PLAIN = {"Besulix": besulix_plain, "Golepel": golepel_plain, "Lutovik": lutovik_plain, "Vogunex": vogunex_plain}
 
 
 # ---- cases: `m` is (model, cfg, pcfg, pw, tol) ------------------------------------------------------------------------

@@ -68,8 +68,9 @@ def causal_conv(stream, w, state, slot_ids, cu_rows, row_seq, out_dtype, residua
 
 
 def latent_prepare(proj, H, dn, dr, R, gain, eps, inv_freq, rot, row_seq, row_pos, new_len, table, pool, rows_cap,
-                   own=True, out_dtype=None):
-    """proj [M, H (dr + dn) (+ dr + R)]: per head [rotated | unrotated] query parts, then [key part | latent].
+                   own=True, out_dtype=None, tail=None, write=True):
+    """proj [M, H (dr + dn) (+ dr + R)]: per head [rotated | unrotated] query parts, then [key part | latent] (or these as
+    rows of their own, `tail`).  write False: the step's rows are returned, not cached.
     Returns q [M, H (dr + R)] with every head's first dr elements set (the rotated query part; the rest is for
     `head_linear`), and the step's rows [rope(key part) | rmsnorm(latent) * gain] (None when own is false), which are
     also written into the cache."""
@@ -80,12 +81,13 @@ def latent_prepare(proj, H, dn, dr, R, gain, eps, inv_freq, rot, row_seq, row_po
     q[:, :, :dr] = _rotate(qr, row_pos, inv_freq, rot).to(out_dtype)
     mine = None
     if own:
-        tail = proj[:, H * (dr + dn):].float()
+        tail = proj[:, H * (dr + dn):].float() if tail is None else tail.float()
         r = _rotate(tail[:, None, :dr], row_pos, inv_freq, rot)[:, 0]
         c = tail[:, dr:]
         c = c * torch.rsqrt((c * c).mean(-1, keepdim=True) + eps) * gain
         mine = torch.cat([r, c], dim=-1).to(out_dtype)
-        _cache_rows(mine, mine, row_seq, row_pos, new_len, table, pool, pool, rows_cap)
+        if write:
+            _cache_rows(mine, mine, row_seq, row_pos, new_len, table, pool, pool, rows_cap)
     return q.reshape(m, H * (dr + R)), mine
 
 
@@ -357,7 +359,7 @@ def ssd_scan(xbc, z, dt, dt_bias, a_log, skip, state, slot_ids, cu_rows, max_cou
     return y.reshape(m, inner) * (zf * torch.sigmoid(zf))
 
 
-def shift_mix(x, mu, state, slot_ids, cu_rows, row_seq, one_row_each=False):
+def shift_mix(x, mu, state, slot_ids, cu_rows, row_seq, one_row_each=False, out_dtype=None):
     """out[s, r] = x[r] + (x[r - 1] - x[r]) * mu[s] within each sequence; the row before a sequence's first row of the
     step is state[slot] (float32 [slots, D]), which then takes the sequence's last row."""
     xf = x.float()
@@ -367,7 +369,7 @@ def shift_mix(x, mu, state, slot_ids, cu_rows, row_seq, one_row_each=False):
         before[a] = state[slot]
         before[a + 1:b] = xf[a:b - 1]
         state[slot] = xf[b - 1]
-    return (xf[None] + (before - xf)[None] * mu[:, None, :]).to(x.dtype)
+    return (xf[None] + (before - xf)[None] * mu[:, None, :]).to(out_dtype or x.dtype)
 
 
 def unary_(x, name):
@@ -440,6 +442,101 @@ def pair_norm_mean(a, b, gain_a, gain_b, eps):
 def mul_sigmoid(x, g):
     x.copy_((x.float() * torch.sigmoid(g.float())).to(x.dtype))
     return x
+
+
+def mul_sigmoid_heads(x, g, heads):
+    m = x.shape[0]
+    x.copy_((x.float().reshape(m, heads, -1) * torch.sigmoid(g.float())[:, :, None]).reshape(m, -1).to(x.dtype))
+    return x
+
+
+def bias_act(rows, bias, activation, out_dtype):
+    y = rows.float() + (bias.float() if bias is not None else 0.0)
+    if activation == "gelu_erf":
+        y = 0.5 * y * (1.0 + torch.erf(y * 0.7071067811865476))
+    else:
+        assert activation is None
+    return y.to(out_dtype)
+
+
+def qkv_prepare(x, bias, H, KV, row, dim, inv_freq, rotary_dim, row_pos, unit_eps, out_dtype, pairing="halves"):
+    m = x.shape[0]
+    y = x.float() + (bias.float() if bias is not None else 0.0)
+    y = y.reshape(m, H + 2 * KV, row)
+    qk = _rotate(y[:, :H + KV], row_pos, inv_freq, rotary_dim, pairing)
+    if unit_eps is not None:
+        qk = qk * torch.rsqrt((qk[..., :dim] ** 2).mean(-1, keepdim=True) + unit_eps)
+    qk[..., dim:] = 0.0
+    q = qk[:, :H].reshape(m, H * row).to(out_dtype)
+    if not KV:
+        return q, None, None
+    return q, qk[:, H:].reshape(m, KV * row).to(out_dtype), y[:, H + KV:].reshape(m, KV * row).to(out_dtype)
+
+
+def pool_write(k, v, KV, row, block, cu_rows, max_count, new_len, slot_ids, sums, table, k_blocks, v_blocks):
+    page = k_blocks.shape[2]
+    for i in range(len(cu_rows) - 1):
+        a, b, slot = int(cu_rows[i]), int(cu_rows[i + 1]), int(slot_ids[i])
+        start = int(new_len[i]) - (b - a)
+        for r in range(a, b):
+            p = start + r - a
+            if p % block == 0:
+                sums[slot].zero_()
+            sums[slot, 0] += k[r].float()
+            sums[slot, 1] += v[r].float()
+            if p % block == block - 1:
+                n = p // block
+                pg = int(table[i, n // page])
+                assert pg >= 0
+                k_blocks[pg, :, n % page, :] = (sums[slot, 0] / block).reshape(KV, row).to(k_blocks.dtype)
+                v_blocks[pg, :, n % page, :] = (sums[slot, 1] / block).reshape(KV, row).to(v_blocks.dtype)
+
+
+def attention_pooled(q, k, v, H, KV, hd, cu_rows, row_seq, row_pos, new_len, table, k_pool, v_pool, rows_cap, scale, softcap,
+                     window, blocks=None, all_values=False):
+    m, page = q.shape[0], k_pool.shape[2]
+    VG = KV if all_values else 1
+    out = torch.zeros((m, H, VG, hd), dtype=torch.float32, device=q.device)
+    qf, kf, vf = q.float().reshape(m, H, hd), k.float().reshape(m, KV, hd), v.float().reshape(m, KV, hd)
+    for i in range(len(cu_rows) - 1):
+        a, b = int(cu_rows[i]), int(cu_rows[i + 1])
+        start = int(new_len[i]) - (b - a)
+        for r in range(a, b):
+            p = start + r - a
+            lo = max(0, p - window + 1) if window else 0
+            keys, vals = [], []
+            if blocks is not None:
+                block, btable, kb, vb = blocks
+                for n in range(max(0, p - window + 1) // block):
+                    pg = int(btable[i, n // page])
+                    keys.append(kb[pg, :, n % page, :].float())
+                    vals.append(vb[pg, :, n % page, :].float())
+            for t in range(lo, p + 1):
+                if t < start:
+                    rr = t % rows_cap if rows_cap else t
+                    pg = int(table[i, rr // page])
+                    keys.append(k_pool[pg, :, rr % page, :].float())
+                    vals.append(v_pool[pg, :, rr % page, :].float())
+                else:
+                    keys.append(kf[a + t - start])
+                    vals.append(vf[a + t - start])
+            keys, vals = torch.stack(keys), torch.stack(vals)            # [n, KV, hd]
+            for h in range(H):
+                g = h // (H // KV)
+                s_ = (keys[:, g] @ qf[r, h]) * scale
+                if softcap:
+                    s_ = softcap * torch.tanh(s_ / softcap)
+                w = torch.softmax(s_, dim=0)
+                for c in range(VG):
+                    out[r, h, c] = w @ vals[:, c if all_values else g]
+    return out
+
+
+def talk_mix(a, talk, out_dtype):
+    m, H, VG, hd = a.shape
+    own = torch.arange(H) // (H // VG)
+    picked = a[:, :, own, :]                              # [m, g, h, hd]: head g's weights on the values of h's kv head
+    return torch.einsum("hg,mghd->mhd", talk.float(), picked).reshape(m, H * hd).to(out_dtype)
 
 
 def gather_rows(x, rows):

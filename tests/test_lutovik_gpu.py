@@ -60,7 +60,8 @@ def run_mixers(rt, mixers, seqs, steps, page=16):
     {id: [per mixer: rows [n, WIDTH]]}."""
     specs = [m.cache_spec() if owner == i else None for i, (m, owner) in enumerate(mixers)]
     states = [{"mixer." + k: v for k, v in m.state_specs().items()} for m, _ in mixers]
-    cache = ModelCache(specs, 4096, 4096, 8, page, rt.dtype, rt.device, entry_states=states)
+    tokens = [{"mixer." + k: v for k, v in m.token_specs().items()} if owner == i else {} for i, (m, owner) in enumerate(mixers)]
+    cache = ModelCache(specs, 4096, 4096, 8, page, rt.dtype, rt.device, entry_states=states, entry_tokens=tokens)
     slots = {i: cache.acquire() for i in seqs}
     done = {i: 0 for i in seqs}
     got = {i: [[] for _ in mixers] for i in seqs}

@@ -350,6 +350,7 @@ extern "C" int tp_add_rms_norm(float* stream, const void* rows, int rows_dtype, 
     if (rows_dtype == TP_BF16 && out_dtype == TP_BF16) rc = add_rms_norm_launch<bf16_t, bf16_t>(stream, rows, n_slices, slice_stride, gain_post, eps_post, gain_next, eps_next, out, M, D, groups, s);
     else if (rows_dtype == TP_F32 && out_dtype == TP_F32) rc = add_rms_norm_launch<float, float>(stream, rows, n_slices, slice_stride, gain_post, eps_post, gain_next, eps_next, out, M, D, groups, s);
     else if (rows_dtype == TP_F32 && out_dtype == TP_BF16) rc = add_rms_norm_launch<float, bf16_t>(stream, rows, n_slices, slice_stride, gain_post, eps_post, gain_next, eps_next, out, M, D, groups, s);
+    else if (rows_dtype == TP_BF16 && out_dtype == TP_F32) rc = add_rms_norm_launch<bf16_t, float>(stream, rows, n_slices, slice_stride, gain_post, eps_post, gain_next, eps_next, out, M, D, groups, s);
     else return tp_fail("add_rms_norm: unsupported dtypes rows %d -> out %d", rows_dtype, out_dtype);
     if (rc) return rc;
     return tp_check_launch("add_rms_norm");
