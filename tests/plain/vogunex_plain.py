@@ -56,12 +56,8 @@ def pooled_window_weights(q, k, scale, softcap, size, pool):
     s = torch.cat([q @ kb.T, q @ k.T], dim=1) * scale
     if softcap:
         s = softcap * torch.tanh(s / softcap)
-    seen = torch.zeros(n, nb + n, dtype=torch.bool)
-    for i in range(n):
-        for b in range(nb):
-            seen[i, b] = b * pool + pool - 1 <= i - size
-        for j in range(n):
-            seen[i, nb + j] = 0 <= i - j < size
+    i, j, b = torch.arange(n)[:, None], torch.arange(n)[None], torch.arange(nb)[None]
+    seen = torch.cat([b * pool + pool - 1 <= i - size, (i - j >= 0) & (i - j < size)], dim=1)       # blocks, then tokens
     w = torch.softmax(s.masked_fill(~seen, -math.inf), dim=1)
     return w[:, :nb], w[:, nb:]
 

@@ -493,7 +493,7 @@ def pool_write(k, v, KV, row, block, cu_rows, max_count, new_len, slot_ids, sums
 
 
 def attention_pooled(q, k, v, H, KV, hd, cu_rows, row_seq, row_pos, new_len, table, k_pool, v_pool, rows_cap, scale, softcap,
-                     window, blocks=None, all_values=False):
+                     window, blocks=None, all_values=False, max_count=None):
     m, page = q.shape[0], k_pool.shape[2]
     VG = KV if all_values else 1
     out = torch.zeros((m, H, VG, hd), dtype=torch.float32, device=q.device)

@@ -64,6 +64,25 @@ def test_pooled_attention_part(rt, H, G, dim, vdim, rot, size, pool, cap):
         assert rel_l2(got[i][0], plain.attention(wide[i], W, "", sizes, EPS)) < tolerance(rt), i
 
 
+@pytest.mark.parametrize("H,G,dim,vdim,size,pool", [(8, 4, 256, 256, 300, 8), (4, 2, 128, 64, 129, 16), (2, 1, 64, 32, 1000, None), (6, 3, 32, 96, 64, 1)])
+def test_matrix_core_kernel_over_many_chunks(H, G, dim, vdim, size, pool):
+    """Sequences long enough for every wave of a block to take several chunks of keys, pooled blocks by the dozen: the
+    matrix-core kernel against the plain implementation, and against the plain kernel on the same rows."""
+    rt = Runtime(dtype="bfloat16", device=DEV)
+    part, W, sizes = pooled_attention(rt, H, G, dim, vdim, 32, size, pool, 25.0, scale=0.5)
+    seqs, wide = sequences(rt, 59, lens={0: 700, 1: 180})
+    steps = [{0: 500, 1: 100}, {0: 1, 1: 1}, {0: 150, 1: 2}] + [{0: 1, 1: 1}] * 49 + [{1: 28}]
+    got = run_mixers(rt, [(part, 0)], seqs, steps, page=64)
+    rt.ops.force_plain_attention = True
+    try:
+        slow = run_mixers(rt, [(part, 0)], seqs, steps, page=64)
+    finally:
+        rt.ops.force_plain_attention = False
+    for i in seqs:
+        assert rel_l2(got[i][0], plain.attention(wide[i], W, "", sizes, EPS)) < tolerance(rt), i
+        assert rel_l2(got[i][0], slow[i][0]) < 4e-3, i
+
+
 def rows_differ(a, b):
     return float(((a - b).norm(dim=1) / b.norm(dim=1)).max())
 

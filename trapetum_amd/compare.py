@@ -1,7 +1,7 @@
-"""Two designs side by side at equal layer sizes: Golepel or Lutovik next to Gemma-2, Besulix next to Lutovik, random
-weights, one MI355X.
+"""Two designs side by side at equal layer sizes: Golepel or Lutovik next to Gemma-2, Besulix or Vogunex next to Lutovik,
+random weights, one MI355X.
 
-    python bench.py --compare golepel|lutovik|besulix [--sizes 2b|9b] [--layers L] [--steps K] [--warmup W]
+    python bench.py --compare golepel|lutovik|besulix|vogunex [--sizes 2b|9b] [--layers L] [--steps K] [--warmup W]
 
 For each design: tokens per second of a prefill of 2,048 tokens and of the generation loop's decode steps at batch 8
 and 1 (HIP graphs, greedy choice on the device), and the time of the kernels a step spends its time in, one by one at
@@ -21,6 +21,12 @@ The Besulix sizes: the same width, vocabulary and number of layers; layers alter
 dense feed-forward of Gemma's width (left: 16 heads on 4 kv heads of 128, values of 128, a rotation of 64 elements,
 chunks of 1,024 positions; right: time-mixing heads of 64 channels filling the width) and a matrix-memory layer without
 a feed-forward (heads of 128 key and 256 value elements filling the width) (`time_besulix_kernels`).
+The Vogunex sizes: the same width, vocabulary and number of layers; of every four layers the first is an attention layer
+(Gemma-2's heads; a window of 1,024 positions, pooled blocks of 16, a score cap, talking heads) with a biased dense
+feed-forward of Gemma's width, the second an attention through a latent (16 heads of 128 + 64, values of 128, a latent
+of 192, a query latent of 768, a window of 1,024, gated heads), the third runs on the first one's weights, the fourth is
+a state-space layer of Lutovik's sizes; the second and fourth have 8 experts of half the dense width, 2 chosen, and a
+gated shared expert of a quarter of it (`time_vogunex_kernels`).
 """
 import json
 import sys
@@ -83,6 +89,180 @@ def besulix_config(which, layers=0):
     mem = {"type": "mlstm", "mixer": {"heads": D // 256, "dim": 128, "vdim": 256, "gate_cap": 15.0}, "mlp": None}
     return BesulixConfig.from_dict({"architecture": "Besulix", "vocab": g["vocab_size"], "width": D, "norm": {"eps": 1e-6},
                                     "logit_softcap": 30.0, "layers": [par if i % 2 == 0 else mem for i in range(n)]})
+
+
+def vogunex_config(which, layers=0):
+    from .config import VogunexConfig
+    g = dict(SIZES, **OTHER_SIZES[which])
+    n = layers or g["num_hidden_layers"]
+    D, I, H, KV, hd = g["hidden_size"], g["intermediate_size"], g["num_attention_heads"], g["num_key_value_heads"], g["head_dim"]
+    att = {"heads": H, "kv_heads": KV, "dim": hd, "vdim": hd, "scale": hd ** -0.5, "softcap": 50.0, "rot": {"base": 10000.0, "dims": 64},
+           "mask": {"size": 1024, "pool": 16}}
+    lat = {"heads": 16, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 192, "q_rank": 768, "scale": 192 ** -0.5,
+           "rot": {"base": 10000.0, "dims": 64}, "mask": {"size": 1024}}
+    ssm = {"heads": D // 64, "vdim": 64, "state": 128, "groups": 4, "conv": 4, "norm_groups": 4}
+    moe = {"kind": "moe", "expert": {"ff": I // 2, "limit": 7.0}, "router": {"experts": 8, "top": 2}, "shared": {"ff": I // 4, "limit": 7.0}}
+    dense = {"kind": "dense", "ff": I}
+    out = []
+    for i in range(n):
+        if i % 4 == 0:
+            out.append({"type": "attention", "mixer": att, "mlp": dense})
+        elif i % 4 == 1:
+            out.append({"type": "latent_attention", "mixer": lat, "mlp": moe})
+        elif i % 4 == 2:
+            out.append({"type": "attention", "mixer": att, "mlp": dense, "weights_of": i - 2})
+        else:
+            out.append({"type": "mamba2", "mixer": ssm, "mlp": moe})
+    return VogunexConfig.from_dict({"architecture": "Vogunex", "vocab": g["vocab_size"], "width": D, "embedding": {"scale": D ** 0.5},
+                                    "norm": {"eps": 1e-6}, "layers": out})
+
+
+def time_vogunex_kernels(engine, cfg, batch, context, prefill_tokens):
+    """Microseconds of Vogunex's kernels at a decode step of `batch` sequences over `context` cached tokens and at a
+    prefill of `prefill_tokens`, each called once per layer on that layer's own weights, replayed from a HIP graph.
+    Products are priced by their weights' bytes (decode) or their flops against the bf16 matrix peak (prefill); the
+    attention over a window and pooled blocks by the keys and values of all kv heads that a query's window and blocks
+    hold (decode) or by the flops of every query head on its own kv head's keys and values (prefill: what it computes
+    beyond that for the mix of the heads is not counted as work)."""
+    import torch
+    from .engine.batch import StepContext
+    model, ops, dev = engine.model, engine.model.rt.ops, engine.model.rt.device
+    bf, f32 = torch.bfloat16, torch.float32
+    blocks = [l.block for l in model.layers]
+    att = [b for b in blocks if hasattr(b.mixer, "talk")]
+    lat = [b for b in blocks if hasattr(b.mixer, "w_absorb")]
+    dense = [b for b in blocks if hasattr(b.feed_forward, "b_up")]
+    moe = [b for b in blocks if hasattr(b.feed_forward, "w_router")]
+    D = cfg.hidden_size
+    out = {}
+    timed = _timer(dev, out)
+    cache = engine.cache
+    entry = lambda group: next(i for i, e in enumerate(model.schedule) if model.layers[e.layer].block is group[0])
+    elems = lambda w: float(w.numel())
+    for rows, tag in ((batch, f"decode_b{batch}"), (prefill_tokens, f"prefill_{prefill_tokens}")):
+        decode = rows == batch
+        slots = [cache.acquire() for _ in range(batch if decode else 1)]
+        try:
+            for s in slots:
+                cache.grow(s, context if decode else rows)
+            counts = [1] * batch if decode else [rows]
+            starts = [context - 1] * batch if decode else [0]
+            ctx = StepContext(model.rt, cache, slots, counts, starts, [])
+            x = torch.randn((rows, D), device=dev).to(bf)
+            one = lambda f, **kw: timed(f"{tag}.{kw.pop('name')}", f, **kw)
+            prod = (lambda name, calls, w, m=rows: one(calls, name=name, bytes_each=2.0 * elems(w)) if decode
+                    else one(calls, name=name, flops_each=2.0 * m * elems(w)))
+            stream = torch.randn((rows, D), device=dev)
+            shift_state = cache.entry_state(0, "token_shift")
+            one([lambda: ops.shift_mix(stream, blocks[0].shift_weight, shift_state, ctx.slot_ids, ctx.cu_rows, ctx.row_seq, one_row_each=decode,
+                                       out_dtype=bf)] * 16, name="token_shift", bytes_each=rows * D * 6.0)
+            if att:
+                e = entry(att)
+                ctx.entry = ctx.cache_owner = e
+                a = att[0].mixer
+                H, KV, row, W, P = a.num_heads, a.num_kv_heads, a.row, a.window, a.pool
+                site, bsite = cache.site(e), cache.entry_site(e, "mixer.blocks")
+                table, btable = ctx.page_table(site.group_index), ctx.page_table(bsite.group_index)
+                kp, vp, cap = site.tensor("k"), site.tensor("v"), site.rows_cap or 0
+                kb, vb, sums = bsite.tensor("k"), bsite.tensor("v"), cache.entry_state(e, "mixer.block_sums")
+                prod("qkv_f32", [(lambda b=b: ops.linear(x, b.mixer.w_qkv, f32)) for b in att], a.w_qkv)
+                qkv = torch.randn((rows, (H + 2 * KV) * row), device=dev)
+                prep = lambda: ops.qkv_prepare(qkv, a.b_qkv, H, KV, row, a.head_dim, a.inv_freq, a.position.rotary_dim, ctx.row_pos,
+                                               a.unit_norm_eps, bf)
+                one([prep] * 16, name="qkv_prepare", bytes_each=rows * (H + 2 * KV) * row * 6.0)
+                q, k, v = prep()
+                one([lambda: ops.pool_write(k, v, KV, row, P, ctx.cu_rows, ctx.max_count, ctx.new_len, ctx.slot_ids, sums, btable, kb, vb)] * 16,
+                    name="pool_write", bytes_each=rows * 2 * KV * row * (2.0 + 2.0 / P))
+                att_call = lambda: ops.attention_pooled(q, k, v, H, KV, row, ctx.cu_rows, ctx.row_seq, ctx.row_pos, ctx.new_len, table, kp, vp, cap,
+                                                        a.query_scale, a.softcap, W, blocks=(P, btable, kb, vb), all_values=True,
+                                                        max_count=ctx.max_count)
+                if decode:
+                    keys = min(context, W) + max(0, context - W) // P
+                    one([att_call] * 8, name=f"attention_{keys}_keys_of_{context}", bytes_each=2.0 * batch * keys * 2 * KV * row)
+                else:
+                    pairs = sum(min(p + 1, W) + max(0, p - W + 1) // P for p in range(rows))
+                    one([att_call] * 4, name=f"attention_window_{W}_blocks_of_{P}", flops_each=4.0 * pairs * H * row)
+                heads = att_call()
+                one([lambda: ops.talk_mix(heads, a.talk, bf)] * 16, name="talk_mix", bytes_each=rows * H * row * (4.0 * KV + 2.0))
+                one([lambda: ops.kv_write(k, v, KV, row, ctx.row_seq, ctx.row_pos, ctx.new_len, table, kp, vp, cap)] * 16, name="kv_write",
+                    bytes_each=rows * 2 * KV * row * 4.0)
+                xa = torch.randn((rows, H * row), device=dev).to(bf)
+                prod("o", [(lambda b=b: ops.linear(xa, b.mixer.w_o, bf, defer=True)) for b in att], a.w_o)
+            if lat:
+                e = entry(lat)
+                ctx.entry = ctx.cache_owner = e
+                mx = lat[0].mixer
+                H, dn, dr, dv, R, lrow = mx.num_heads, mx.nope_dim, mx.rope_dim, mx.value_dim, mx.rank, mx.row
+                site = cache.site(e)
+                table, pool, cap = ctx.page_table(site.group_index), site.tensor("latent"), site.rows_cap or 0
+                prod("latent_dq_f32", [(lambda b=b: ops.linear(x, b.mixer.w_dq, f32)) for b in lat], mx.w_dq)
+                cq = torch.randn((rows, mx.query_rank), device=dev).to(bf)
+                prod("latent_uq", [(lambda b=b: ops.linear(cq, b.mixer.w_uq, bf)) for b in lat], mx.w_uq)
+                prod("latent_dkv", [(lambda b=b: ops.linear(x, b.mixer.w_tail, bf)) for b in lat], mx.w_tail)
+                proj, tail = ops.linear(cq, mx.w_uq, bf), ops.linear(x, mx.w_tail, bf)
+                prep = lambda: ops.latent_prepare(proj, H, dn, dr, R, mx.latent_gain, 1e-6, mx.inv_freq, mx.position.rotary_dim, ctx.row_seq,
+                                                  ctx.row_pos, ctx.new_len, table, pool, cap, own=True, out_dtype=bf, tail=tail)
+                one([prep] * 16, name="latent_prepare", bytes_each=rows * (proj.shape[1] + H * dr + 3 * lrow) * 2.0)
+                q, mine = prep()
+                xq = proj.view(rows, H, dr + dn)[:, :, dr:]
+                qv = q.view(rows, H, lrow)[:, :, dr:]
+                one([(lambda b=b: ops.head_linear(xq, b.mixer.w_absorb, qv)) for b in lat], name="latent_absorb",
+                    bytes_each=2.0 * (elems(mx.w_absorb) + rows * H * (dn + R)))
+                if decode:
+                    keys = min(context, mx.window)
+                    per = next(g for g in (mx.DECODE_GROUP_LONG if keys >= mx.LONG_KEYS else mx.DECODE_GROUP, 4, 2, 1) if H % g == 0)
+                    one([lambda: ops.attention_decode(q, H, 1, lrow, ctx.new_len, table, pool, pool, cap, mx.scale, 0.0, mx.window, bf,
+                                                      max_keys=ctx.max_rows_visible(site), head_groups=H // per,
+                                                      splits=ops.decode_splits(batch * (H // per), 1, lrow, keys))] * 8,
+                        name=f"latent_attention_{keys}_keys", bytes_each=2.0 * batch * keys * lrow)
+                else:
+                    pairs = sum(min(p + 1, mx.window) for p in range(rows))
+                    one([lambda: ops.attention_prefill(q, mine, mine, H, 1, lrow, ctx.cu_rows, rows, mx.scale, 0.0, mx.window, bf,
+                                                       row_seq=ctx.row_seq, row_pos=ctx.row_pos, wide_weights=True)] * 4,
+                        name=f"latent_attention_window_{mx.window}", flops_each=4.0 * pairs * H * lrow)
+                o_lat = torch.randn((rows, H * lrow), device=dev).to(bf)
+                ov = o_lat.view(rows, H, lrow)[:, :, dr:]
+                one([(lambda b=b: ops.head_linear(ov, b.mixer.w_up, None)) for b in lat], name="latent_up",
+                    bytes_each=2.0 * (elems(mx.w_up) + rows * H * (R + dv)))
+                hv = torch.randn((rows, H * dv), device=dev).to(bf)
+                gates = torch.randn((rows, H), device=dev)
+                one([lambda: ops.mul_sigmoid_heads(hv, gates, H)] * 16, name="gate_heads", bytes_each=rows * H * dv * 4.0)
+                prod("latent_o", [(lambda b=b: ops.linear(hv, b.mixer.w_o, bf, defer=True)) for b in lat], mx.w_o)
+            if dense:
+                ff = dense[0].feed_forward
+                prod("up_f32", [(lambda b=b: ops.linear(x, b.feed_forward.w_up, f32)) for b in dense], ff.w_up)
+                up = torch.randn((rows, ff.intermediate_size), device=dev)
+                one([lambda: ops.bias_act(up, ff.b_up, "gelu_erf", bf)] * 16, name="bias_gelu", bytes_each=rows * ff.intermediate_size * 6.0)
+                xi = torch.randn((rows, ff.intermediate_size), device=dev).to(bf)
+                prod("down_bias_f32", [(lambda b=b: ops.linear(xi, b.feed_forward.w_down, f32, bias=b.feed_forward.b_down)) for b in dense], ff.w_down)
+            if moe:
+                ff = moe[0].feed_forward
+                logits = torch.randn((rows, ff.n_experts), device=dev)
+                chosen, weights = ops.route_top(logits, ff.top, True)
+                one([lambda: ops.route_top(logits, ff.top, True)] * 16, name="route_top")
+                used = len(set(chosen.reshape(-1).tolist()))
+                per_expert = float(ff.w_gate_up[0].numel() + ff.w_down[0].numel())
+                calls = [(lambda b=b: ops.expert_ffn(x, chosen, weights, b.feed_forward.w_gate_up, b.feed_forward.w_down, ff.limit, ff.gate_alpha,
+                                                     ff.up_shift)) for b in moe]
+                if decode:
+                    one(calls, name=f"experts_{used}_used", bytes_each=2.0 * used * per_expert)
+                else:
+                    one(calls, name="experts", flops_each=2.0 * rows * ff.top * per_expert)
+                sh = ff.shared
+                prod("shared_gate_up", [(lambda b=b: ops.gated_linear(x, b.feed_forward.shared.w_gate_up, sh.intermediate_size, "quick_gelu", bf,
+                                                                      limit=sh.limit, up_shift=sh.up_shift)) for b in moe],
+                     sh.w_gate_up[:2 * sh.intermediate_size])
+                both = torch.randn((rows, D), device=dev)
+                sg = torch.randn((rows, 1), device=dev)
+                one([lambda: ops.mul_sigmoid_heads(both, sg, 1)] * 16, name="gate_shared", bytes_each=rows * D * 8.0)
+            rows_b = torch.randn((rows, D), device=dev).to(bf)
+            g = torch.ones(D, device=dev)
+            one([lambda: ops.add_rms_norm(stream, rows_b, None, 0.0, g, 1e-6, f32)] * 16, name="add_rms_norm_f32",
+                bytes_each=rows * D * (4 + 4 + 2 + 4) + 4.0 * D)
+        finally:
+            for s in slots:
+                cache.release(s)
+    return out
 
 
 def gemma_config(which, layers=0):
@@ -568,9 +748,10 @@ def main(args):
     prompt, batch = args.prompt, args.batch
     design = args.compare
     build, time_design = {"golepel": (golepel_config, time_golepel_kernels), "lutovik": (lutovik_config, time_lutovik_kernels),
-                          "besulix": (besulix_config, time_besulix_kernels)}[design]
+                          "besulix": (besulix_config, time_besulix_kernels), "vogunex": (vogunex_config, time_vogunex_kernels)}[design]
     # the design it stands next to: the closest of the others
-    other, build_other, time_other, title = {"besulix": ("lutovik", lutovik_config, time_lutovik_kernels, "Lutovik")}.get(
+    beside_lutovik = ("lutovik", lutovik_config, time_lutovik_kernels, "Lutovik")
+    other, build_other, time_other, title = {"besulix": beside_lutovik, "vogunex": beside_lutovik}.get(
         design, ("gemma2", gemma_config, time_kernels, "Gemma-2"))
     line = {"metric": f"{design.capitalize()} next to {title} at {which} layer sizes: prefill and decode tok/s", "unit": "tok/s", "n_gpus": 1,
             "steps": steps, "warmup": warmup, "dtype": "bf16", "data": "synthetic: seeded random weights N(0, 0.02) and uniform-random token ids",

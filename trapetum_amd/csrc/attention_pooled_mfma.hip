@@ -1,0 +1,252 @@
+// Matrix-core kernel of the attention over a window plus pooled blocks (see attention_pooled.hip for the mechanism and
+// the plain kernel), for bf16 rows of TP_HD elements, TP_HD a multiple of 32 up to 256.  One launch serves prompts,
+// portions of prompts and decode steps.
+//
+// A block of four waves owns 16 consecutive query rows of one sequence, one query head g and one kv head c whose
+// values g's weights are applied to.  The keys the 16 queries can see are one list, the pooled blocks 0 .. NB - 1 (NB of
+// the tile's last query) and then the positions from the first query's window start to the last query; each query masks
+// what it does not see.  The list is cut into chunks of 32 keys that the waves take in turn, every wave with its own
+// running maximum, sum and outputs, which meet in LDS once at the end, in wave order.
+//
+// Scores transposed, S^T = K Q^T, with `v_mfma_f32_16x16x32_bf16`: the A operand is 16 key rows straight from global
+// memory (cache pages, pooled pages or the step's rows: a lane computes one key's address and hands it on by lane
+// reads), the B operand the queries in registers; a lane gets four keys of one query, so the softmax statistics are
+// per-lane scalars and two lane exchanges.  A lane's eight weights of a chunk (two score tiles) are the B operand of the
+// second product as they lie, O^T = V^T P^T; the order of the 32 keys in that product's K dimension is then (4j + i of
+// the first tile, 4j + i of the second) for lane group j, and V^T is read from an LDS copy of the chunk's value rows
+// in that order.  The weights enter the second product as two bf16 terms (a weight's rounding and the rounding's
+// remainder), so they meet the values with 16 bits of mantissa.  Elements of a head are visited in the order
+// (j, step) -> j HD / 4 + 8 step for queries and keys alike, so that a lane reads one contiguous quarter of a key row.
+#include "common.h"
+
+#ifndef TP_HD
+#error "compile with -DTP_HD=<head size>"
+#endif
+
+#if TP_HD % 32 == 0
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 pt_bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float pt_f32x4;
+union PtFrag { uint4 u; pt_bf16x8 v; bf16_t h[8]; };
+
+struct AttnPooledTileArgs {
+    const bf16_t* q; long q_stride;
+    const bf16_t* k; long k_stride; const bf16_t* v; long v_stride;
+    const int* cu_rows; const int* new_len;
+    const int* table; int table_w; const bf16_t* k_pool; const bf16_t* v_pool; int page; int rows_cap;
+    const int* ptable; int ptable_w; const bf16_t* pk; const bf16_t* pv; int P;
+    float* out;
+    int H, KV, VG; float scale, cap; int window;
+};
+
+namespace {
+constexpr int HD = TP_HD, WAVES = 4, CHUNK = 32, KS = HD / 32, VT = HD / 16, VSTRIDE = HD + 8, PIECES = HD / 8;
+constexpr int STAGE_BYTES = WAVES * CHUNK * VSTRIDE * 2, MERGE_BYTES = WAVES * HD * 16 * 4;
+constexpr int LDS_BYTES = STAGE_BYTES > MERGE_BYTES ? STAGE_BYTES : MERGE_BYTES;
+
+__device__ __forceinline__ const bf16_t* lane_ptr(const bf16_t* p, int lane) {
+    const uint64_t x = (uint64_t)p;
+    const uint32_t lo = __shfl((int)(uint32_t)x, lane, 64), hi = __shfl((int)(uint32_t)(x >> 32), lane, 64);
+    return (const bf16_t*)(((uint64_t)hi << 32) | lo);
+}
+}
+
+__global__ void __launch_bounds__(256)
+attn_pooled_tile_k(AttnPooledTileArgs a) {
+    __shared__ __attribute__((aligned(16))) unsigned char lds[LDS_BYTES];
+    __shared__ float m_s[WAVES][16], l_s[WAVES][16];
+    const int tile = blockIdx.x, seq = blockIdx.y, h = blockIdx.z / a.VG, c = blockIdx.z - h * a.VG;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, col = lane & 15, j = lane >> 4;
+    const int first_row = a.cu_rows[seq], count = a.cu_rows[seq + 1] - first_row;
+    if (tile * 16 >= count) return;
+    const int gk = h / (a.H / a.KV), gv = a.VG > 1 ? c : gk;
+    const int start = a.new_len[seq] - count;             // the first position that is a row of the step
+    const int r0 = tile * 16, nq = min(16, count - r0);
+    const int p0 = start + r0, p_max = p0 + nq - 1;
+    const int W = a.window;
+    const int LO = W > 0 ? max(0, p0 - W + 1) : 0;
+    const int NB = a.P > 0 ? max(0, p_max - W + 1) / a.P : 0;
+    const int n_keys = NB + (p_max - LO + 1);
+    const int qc = min(col, nq - 1), pq = p0 + qc;         // this lane's query (a column of the score tiles)
+    const int my_lo = W > 0 ? max(0, pq - W + 1) : 0, my_nb = a.P > 0 ? max(0, pq - W + 1) / a.P : 0;
+
+    PtFrag qf[KS];
+    {
+        const bf16_t* qrow = a.q + (size_t)(first_row + r0 + qc) * a.q_stride + (size_t)h * HD + j * (HD / 4);
+#pragma unroll
+        for (int s = 0; s < KS; s++) qf[s].u = *reinterpret_cast<const uint4*>(qrow + s * 8);
+    }
+    pt_f32x4 acc[VT];
+#pragma unroll
+    for (int t = 0; t < VT; t++) acc[t] = (pt_f32x4){0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.f;
+    bf16_t* v_lds = reinterpret_cast<bf16_t*>(lds) + (size_t)wave * CHUNK * VSTRIDE;
+    const float soc = a.cap > 0.f ? a.scale / a.cap : 0.f;
+
+    for (int u0 = wave * CHUNK; u0 < n_keys; u0 += WAVES * CHUNK) {
+        // ---- where the chunk's 32 keys and values lie: lane l works out key l % 32 -------------------------------------
+        const bf16_t *kp, *vp;
+        {
+            const int u = min(u0 + (lane & 31), n_keys - 1);   // past the last key: a row that exists, masked below
+            if (u < NB) {
+                const int pg = a.ptable[(size_t)seq * a.ptable_w + u / a.page];
+                const size_t at = (size_t)pg * a.KV * a.page + u % a.page;
+                kp = a.pk + (at + (size_t)gk * a.page) * HD;
+                vp = a.pv + (at + (size_t)gv * a.page) * HD;
+            } else {
+                const int t = LO + u - NB;
+                if (t < start) {
+                    const int row = a.rows_cap > 0 ? t % a.rows_cap : t;
+                    const int pg = a.table[(size_t)seq * a.table_w + row / a.page];
+                    const size_t at = (size_t)pg * a.KV * a.page + row % a.page;
+                    kp = a.k_pool + (at + (size_t)gk * a.page) * HD;
+                    vp = a.v_pool + (at + (size_t)gv * a.page) * HD;
+                } else {
+                    const size_t row = (size_t)(first_row + t - start);
+                    kp = a.k + row * a.k_stride + (size_t)gk * HD;
+                    vp = a.v + row * a.v_stride + (size_t)gv * HD;
+                }
+            }
+        }
+        PtFrag kf[2][KS];
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+            const bf16_t* mine = lane_ptr(kp, t * 16 + col) + j * (HD / 4);
+#pragma unroll
+            for (int s = 0; s < KS; s++) kf[t][s].u = *reinterpret_cast<const uint4*>(mine + s * 8);
+        }
+        // the chunk's value rows into this wave's part of LDS, 16 bytes a lane and load
+#pragma unroll
+        for (int i = 0; i < CHUNK * PIECES / 64; i++) {
+            const int idx = lane + 64 * i, key = idx / PIECES, piece = idx - key * PIECES;
+            const uint4 x = *reinterpret_cast<const uint4*>(lane_ptr(vp, key) + piece * 8);
+            *reinterpret_cast<uint4*>(v_lds + key * VSTRIDE + piece * 8) = x;
+        }
+        // ---- scores: two tiles of 16 keys; lane (col, j) gets keys 4j .. 4j + 3 of each for query col ------------------
+        pt_f32x4 sc[2];
+        float pr[2][4];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+            sc[t] = (pt_f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < KS; s++) sc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[t][s].v, qf[s].v, sc[t], 0, 0, 0);
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int u = u0 + t * 16 + j * 4 + i, pos = LO + u - NB;
+                const bool seen = u < n_keys && (u < NB ? u < my_nb : (pos >= my_lo && pos <= pq));
+                const float x = a.cap > 0.f ? a.cap * tanhf(sc[t][i] * soc) : sc[t][i] * a.scale;
+                pr[t][i] = seen ? x : -INFINITY;
+                mx = fmaxf(mx, pr[t][i]);
+            }
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m_run, mx);
+        float alpha = 1.f, psum = 0.f;
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                pr[t][i] = m_new == -INFINITY ? 0.f : expf(pr[t][i] - m_new);
+                psum += pr[t][i];
+            }
+        if (m_new != -INFINITY) alpha = expf(m_run - m_new);
+        psum += __shfl_xor(psum, 16, 64);
+        psum += __shfl_xor(psum, 32, 64);
+        l_run = l_run * alpha + psum;
+        m_run = m_new;
+        PtFrag ph, pl;                                   // the weights as two bf16 terms
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const bf16_t hi = f32_to_bf16(pr[t][i]);
+                ph.h[t * 4 + i] = hi;
+                pl.h[t * 4 + i] = f32_to_bf16(pr[t][i] - bf16_to_f32(hi));
+            }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        // ---- O^T += V^T P^T: lane (col, j) reads element vt * 16 + col of the keys 4j + i of both tiles ---------------------
+#pragma unroll
+        for (int vt = 0; vt < VT; vt++) {
+            PtFrag vf;
+#pragma unroll
+            for (int e = 0; e < 8; e++) vf.h[e] = v_lds[((e < 4 ? 0 : 12) + 4 * j + e) * VSTRIDE + vt * 16 + col];
+            acc[vt] *= alpha;
+            acc[vt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, ph.v, acc[vt], 0, 0, 0);
+            acc[vt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pl.v, acc[vt], 0, 0, 0);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    }
+    // ---- the waves' parts meet, in wave order ------------------------------------------------------------------------------
+    __syncthreads();                                     // every wave is done with its part of LDS
+    float* o_s = reinterpret_cast<float*>(lds);          // [wave][VT][4][64]
+    if (j == 0) { m_s[wave][col] = m_run; l_s[wave][col] = l_run; }
+#pragma unroll
+    for (int vt = 0; vt < VT; vt++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) o_s[((size_t)(wave * VT + vt) * 4 + i) * 64 + lane] = acc[vt][i];
+    __syncthreads();
+    float M = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < WAVES; w++) M = fmaxf(M, m_s[w][col]);
+    float f[WAVES], L = 0.f;
+#pragma unroll
+    for (int w = 0; w < WAVES; w++) {
+        f[w] = m_s[w][col] == -INFINITY ? 0.f : expf(m_s[w][col] - M);
+        L += l_s[w][col] * f[w];
+    }
+    const float inv = 1.f / L;
+    if (col < nq) {
+        float* orow = a.out + (((size_t)(first_row + r0 + col) * a.H + h) * a.VG + c) * HD;
+        for (int vt = wave; vt < VT; vt += WAVES) {
+            float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+            float* oe = reinterpret_cast<float*>(&o);
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                float s = 0.f;
+#pragma unroll
+                for (int w = 0; w < WAVES; w++) s += o_s[((size_t)(w * VT + vt) * 4 + i) * 64 + lane] * f[w];
+                oe[i] = s * inv;
+            }
+            *reinterpret_cast<float4*>(orow + vt * 16 + j * 4) = o;
+        }
+    }
+}
+
+extern "C" int tp_attn_pooled_tile(const void* q, long q_stride, const void* k, long k_stride, const void* v, long v_stride,
+                                   int n_seq, int max_count, int H, int KV, const int* cu_rows, const int* new_len,
+                                   const int* table, int table_w, const void* k_pool, const void* v_pool, int page, int rows_cap,
+                                   const int* ptable, int ptable_w, const void* pk, const void* pv, int P,
+                                   float scale, float cap, int window, int all_values, float* out, void* stream) {
+    TP_REQUIRE(n_seq > 0 && max_count > 0 && H > 0 && KV > 0 && H % KV == 0, "attention (pooled): shape sequences=%d rows=%d heads=%d kv=%d", n_seq, max_count, H, KV);
+    TP_REQUIRE(q && k && v && cu_rows && new_len && out && table && k_pool && v_pool && page > 0 && table_w > 0, "attention (pooled): null operand");
+    TP_REQUIRE(rows_cap >= 0 && (rows_cap == 0 || rows_cap % page == 0), "attention (pooled): ring of %d rows is no multiple of the page size %d", rows_cap, page);
+    TP_REQUIRE(P >= 0 && (P == 0 || (window > 0 && ptable && pk && pv && ptable_w > 0)), "attention (pooled): blocks of %d positions need a window, their page table and pools", P);
+    TP_REQUIRE(q_stride % 8 == 0 && k_stride % 8 == 0 && v_stride % 8 == 0, "attention (pooled): row strides must be whole 16-byte pieces");
+    for (const void* p : {q, k, v, k_pool, v_pool, pk, pv, (const void*)out})
+        TP_REQUIRE((uintptr_t)p % 16 == 0, "attention (pooled): operands must be aligned to 16 bytes");
+    const int VG = all_values ? KV : 1;
+    TP_REQUIRE(n_seq <= 65535 && (long)H * VG <= 65535, "attention (pooled): %d sequences or %d head pairs exceed one launch", n_seq, H * VG);
+    AttnPooledTileArgs a{};
+    a.q = (const bf16_t*)q; a.q_stride = q_stride; a.k = (const bf16_t*)k; a.k_stride = k_stride; a.v = (const bf16_t*)v; a.v_stride = v_stride;
+    a.cu_rows = cu_rows; a.new_len = new_len; a.table = table; a.table_w = table_w; a.k_pool = (const bf16_t*)k_pool; a.v_pool = (const bf16_t*)v_pool;
+    a.page = page; a.rows_cap = rows_cap; a.ptable = ptable; a.ptable_w = ptable_w; a.pk = (const bf16_t*)pk; a.pv = (const bf16_t*)pv; a.P = P;
+    a.out = out; a.H = H; a.KV = KV; a.VG = VG; a.scale = scale; a.cap = cap; a.window = window;
+    dim3 grid(tp_cdiv(max_count, 16), n_seq, H * VG);
+    attn_pooled_tile_k<<<grid, 256, 0, (hipStream_t)stream>>>(a);
+    return tp_check_launch("attention (pooled, matrix cores)");
+}
+
+#else
+
+extern "C" int tp_attn_pooled_tile(const void*, long, const void*, long, const void*, long, int, int, int, int, const int*, const int*,
+                                   const int*, int, const void*, const void*, int, int, const int*, int, const void*, const void*, int,
+                                   float, float, int, int, float*, void*) {
+    return tp_fail("attention (pooled, matrix cores): head size %d is no multiple of 32", TP_HD);
+}
+
+#endif

@@ -20,7 +20,7 @@ FLAGS = ["--offload-arch=" + ARCH, "-O3", "-fPIC", "-std=c++17",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-result"]
 CORE_SOURCES = ["elementwise.hip", "gemm.hip", "gemm_skinny.hip", "gemm_mfma.hip", "gemv.hip", "gemm_rows8.hip", "attention_simple.hip", "sampling.hip", "probes.hip",
                 "conv.hip", "latent.hip", "moe.hip", "ssd.hip", "recurrent.hip", "attention_pooled.hip"]
-ATTN_SOURCES = ["attention_mfma.hip", "attention_prefill.hip"]      # decode steps; steps of many queries
+ATTN_SOURCES = ["attention_mfma.hip", "attention_prefill.hip", "attention_pooled_mfma.hip"]      # decode steps; steps of many queries; a window with pooled blocks
 _NOISE = "is not a recognized feature for this target"
 
 

@@ -68,6 +68,7 @@ _ATTN_SIGS = {
     "tp_attn_decode": [_P, _L, _I, _I, _I, _P, _P, _I, _P, _P, _I, _I, _F, _F, _I, _I, _P, _P, _P, _P, _I, _P],
     "tp_attn_decode_shared": [_P, _L, _I, _I, _I, _I, _P, _P, _I, _P, _P, _I, _I, _F, _F, _I, _P, _P, _I, _P],
     "tp_attn_decode_workspace_floats": [_I, _I, _I],
+    "tp_attn_pooled_tile": [_P, _L, _P, _L, _P, _L, _I, _I, _I, _I, _P, _P, _P, _I, _P, _P, _I, _I, _P, _I, _P, _P, _I, _F, _F, _I, _I, _P, _P],
     "tp_attn_decode_fused": [_P, _I, _I, _L, _L, _P, _I, _I, _I, _I, _I, _P, _P, _I, _P, _P, _I, _I, _F, _F, _I, _P, _P, _I, _P],
 }
 
@@ -808,12 +809,14 @@ class HipOps:
                    k_blocks.data_ptr(), v_blocks.data_ptr(), k_blocks.shape[2], self._stream())
 
     def attention_pooled(self, q, k, v, H, KV, hd, cu_rows, row_seq, row_pos, new_len, table, k_pool, v_pool, rows_cap,
-                         scale, softcap, window, blocks=None, all_values=False):
+                         scale, softcap, window, blocks=None, all_values=False, max_count=None):
         """Attention of the step's queries over the positions their window still holds (those before the step read in
         place from the cache, the step's own rows from k and v) and, with blocks = (block size, page table, key pool,
         value pool), over one pooled key and value per block of positions that lies wholly before the window; one
         softmax over both.  Returns float32 [M, H, KV if all_values else 1, hd]: with all_values every query head's
-        weights are applied to the values of every kv head (what a mix of the heads' weights needs)."""
+        weights are applied to the values of every kv head (what a mix of the heads' weights needs).  max_count: the most
+        rows a sequence brings (a host number; with it bf16 heads of a multiple of 32 elements up to 256 run on the
+        matrix cores)."""
         self._dev(q, k, v, cu_rows, row_seq, row_pos, new_len, table, k_pool, v_pool)
         m = q.shape[0]
         qs, ks, vs = self._rows(q, "attention_pooled q"), self._rows(k, "attention_pooled k"), self._rows(v, "attention_pooled v")
@@ -832,6 +835,14 @@ class HipOps:
             if kb.shape[2] != page or not window:
                 raise KernelError("attention_pooled: the blocks' pools have the cache's page size, and blocks need a window")
         self_out = torch.empty((m, H, KV if all_values else 1, hd), dtype=torch.float32, device=self.device)
+        pieces = all(t is None or (t.data_ptr() % 16 == 0) for t in (q, k, v)) and qs % 8 == 0 and ks % 8 == 0 and vs % 8 == 0
+        if max_count and not self.force_plain_attention and q.dtype == torch.bfloat16 and hd % 32 == 0 and hd <= 256 and pieces:
+            self._call(self.attn_lib(hd), "tp_attn_pooled_tile", q.data_ptr(), qs, k.data_ptr(), ks, v.data_ptr(), vs, n, int(max_count), H, KV,
+                       cu_rows.data_ptr(), new_len.data_ptr(), table.data_ptr(), table.shape[1], k_pool.data_ptr(), v_pool.data_ptr(), page,
+                       rows_cap or 0, btable.data_ptr() if blocks else None, btable.shape[1] if blocks else 0,
+                       kb.data_ptr() if blocks else None, vb.data_ptr() if blocks else None, int(block) if blocks else 0,
+                       float(scale), float(softcap or 0.0), int(window or 0), 1 if all_values else 0, self_out.data_ptr(), self._stream())
+            return self_out
         self._call(self.lib, "tp_attn_pooled", q.data_ptr(), qs, k.data_ptr(), ks, v.data_ptr(), vs, _code(q.dtype), m, H, KV, hd,
                    cu_rows.data_ptr(), row_seq.data_ptr(), row_pos.data_ptr(), new_len.data_ptr(), table.data_ptr(), table.shape[1],
                    k_pool.data_ptr(), v_pool.data_ptr(), page, rows_cap or 0,

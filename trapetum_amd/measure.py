@@ -174,8 +174,8 @@ def main(argv=None):
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the further points (other batches, contexts and sizes) and the kernels' times")
     ap.add_argument("--no-graph", action="store_true", help="launch decode steps kernel by kernel instead of replaying a HIP graph")
-    ap.add_argument("--compare", default=None, choices=["golepel", "lutovik", "besulix"],
-                    help="instead of the metric: that design next to the closest other (Gemma-2; for besulix, Lutovik) at equal layer sizes "
+    ap.add_argument("--compare", default=None, choices=["golepel", "lutovik", "besulix", "vogunex"],
+                    help="instead of the metric: that design next to the closest other (Gemma-2; for besulix and vogunex, Lutovik) at equal layer sizes "
                          "(--sizes 2b or 9b), prefill, decode and kernels")
     args = ap.parse_args(argv)
     if args.gpus != 1:

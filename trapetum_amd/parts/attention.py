@@ -234,7 +234,7 @@ class Attention(Mixer):
             blocks = (self.pool, btable, kb, vb)
         a = ops.attention_pooled(q, k, v, H, KV, hd, ctx.cu_rows, ctx.row_seq, ctx.row_pos, ctx.new_len, table, k_pool, v_pool,
                                  rows_cap, self.query_scale, self.softcap, self.window, blocks=blocks,
-                                 all_values=self.talk_name is not None)
+                                 all_values=self.talk_name is not None, max_count=ctx.max_count)
         out = ops.talk_mix(a, self.talk, ctx.dtype)
         ops.kv_write(k, v, KV, hd, ctx.row_seq, ctx.row_pos, ctx.new_len, table, k_pool, v_pool, rows_cap)
         return self._project_out(ctx, x, out)
