@@ -450,12 +450,16 @@ def mul_sigmoid_heads(x, g, heads):
     return x
 
 
-def bias_act(rows, bias, activation, out_dtype):
+def bias_act(rows, bias, activation, out_dtype, pad=0):
     y = rows.float() + (bias.float() if bias is not None else 0.0)
     if activation == "gelu_erf":
         y = 0.5 * y * (1.0 + torch.erf(y * 0.7071067811865476))
     else:
         assert activation is None
+    if pad:
+        tail = torch.zeros((y.shape[0], pad), dtype=y.dtype, device=y.device)
+        tail[:, 0] = 1.0
+        y = torch.cat([y, tail], dim=1)
     return y.to(out_dtype)
 
 

@@ -114,6 +114,34 @@ def test_a_page_per_block_of_tokens():
         TokenSpec.of(8, every=2, k=(1, 4))
 
 
+def test_a_bias_rides_in_the_matrix_only_where_it_is_exact():
+    """The second product of the biased feed-forward carries its bias as a column of its matrix when the bias has the
+    matrix's width, and adds it in a launch of its own when it does not; both give the same rows."""
+    import types
+
+    from trapetum_amd.registry import build_part
+
+    from .cpu_engine import ref_ops_namespace
+    g = torch.Generator().manual_seed(3)
+    d, f = 24, 40
+    T = {"up": torch.randn(f, d, generator=g).to(torch.bfloat16), "up.b": torch.randn(f, generator=g).to(torch.bfloat16),
+         "down": torch.randn(d, f, generator=g).to(torch.bfloat16), "down.b": torch.randn(d, generator=g).to(torch.bfloat16)}
+    x = torch.randn(7, d, generator=g)
+    rt = types.SimpleNamespace(matrix=lambda t: t.float(), ops=ref_ops_namespace())
+    ctx = types.SimpleNamespace(ops=rt.ops, dtype=torch.float32)
+    outs = []
+    for exact in (True, False):
+        t = dict(T)
+        if not exact:
+            t["down.b"] = T["down.b"].float() + 1e-3            # no bfloat16 number
+        part = build_part("feed_forward", ("biased_mlp", dict(hidden_size=d, intermediate_size=f)))
+        part.bind(t, rt)
+        assert part.folded == exact
+        a = x @ t["up"].float().T + t["up.b"].float()
+        want = (0.5 * a * (1 + torch.erf(a / 2 ** 0.5))) @ t["down"].float().T + t["down.b"].float()
+        assert torch.allclose(rt.ops.rows(part.forward(ctx, x), torch.float32), want, atol=1e-4)
+
+
 def test_whole_and_token_by_token(m):
     mc.whole_and_token_by_token(m, n=45)
 

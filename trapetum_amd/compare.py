@@ -233,8 +233,8 @@ def time_vogunex_kernels(engine, cfg, batch, context, prefill_tokens):
                 prod("up_f32", [(lambda b=b: ops.linear(x, b.feed_forward.w_up, f32)) for b in dense], ff.w_up)
                 up = torch.randn((rows, ff.intermediate_size), device=dev)
                 one([lambda: ops.bias_act(up, ff.b_up, "gelu_erf", bf)] * 16, name="bias_gelu", bytes_each=rows * ff.intermediate_size * 6.0)
-                xi = torch.randn((rows, ff.intermediate_size), device=dev).to(bf)
-                prod("down_bias_f32", [(lambda b=b: ops.linear(xi, b.feed_forward.w_down, f32, bias=b.feed_forward.b_down)) for b in dense], ff.w_down)
+                xi = torch.randn((rows, ff.w_down.shape[1]), device=dev).to(bf)
+                prod("down_with_bias", [(lambda b=b: ops.linear(xi, b.feed_forward.w_down, bf, defer=True)) for b in dense], ff.w_down)
             if moe:
                 ff = moe[0].feed_forward
                 logits = torch.randn((rows, ff.n_experts), device=dev)

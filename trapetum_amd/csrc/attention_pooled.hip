@@ -272,23 +272,24 @@ extern "C" int tp_attn_pooled(const void* q, long q_stride, const void* k, long 
 // a [rows, H, VG, hd] float32 (VG = KV: every head's weights on every kv head's values); out [rows, H, hd]:
 // out_h = sum_g talk[h, g] a[g, kv(h)], the sum in float32 in the order of g.
 template <typename T>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(128)
 talk_mix_k(const float* __restrict__ a, const float* __restrict__ talk, T* __restrict__ out, int H, int KV, int hd) {
-    const int r = blockIdx.x;
-    for (int i = threadIdx.x; i < H * hd; i += 256) {
-        const int h = i / hd, d = i - h * hd, c = h / (H / KV);
+    const int r = blockIdx.x, h = blockIdx.y, c = h / (H / KV);           // grid (rows, heads)
+    const float* src = a + ((size_t)r * H * KV + c) * hd;                  // head g's sums on kv head c: + g KV hd
+    for (int d = threadIdx.x; d < hd; d += 128) {
         float acc = 0.f;
-        for (int g = 0; g < H; g++) acc = __builtin_fmaf(talk[h * H + g], a[(((size_t)r * H + g) * KV + c) * hd + d], acc);
-        st_f32(out + (size_t)r * H * hd + i, acc);
+        for (int g = 0; g < H; g++) acc = __builtin_fmaf(talk[h * H + g], src[(size_t)g * KV * hd + d], acc);
+        st_f32(out + ((size_t)r * H + h) * hd + d, acc);
     }
 }
 
 extern "C" int tp_talk_mix(const float* a, const float* talk, void* out, int out_dtype, int M, int H, int KV, int hd, void* stream) {
     TP_REQUIRE(M > 0 && H > 0 && KV > 0 && hd > 0 && H % KV == 0, "talk_mix: shape rows=%d heads=%d kv=%d head_dim=%d", M, H, KV, hd);
     TP_REQUIRE(a && talk && out, "talk_mix: null operand");
+    TP_REQUIRE(H <= 65535, "talk_mix: %d heads exceed one launch", H);
     hipStream_t s = (hipStream_t)stream;
-    if (out_dtype == TP_BF16) talk_mix_k<bf16_t><<<M, 256, 0, s>>>(a, talk, (bf16_t*)out, H, KV, hd);
-    else if (out_dtype == TP_F32) talk_mix_k<float><<<M, 256, 0, s>>>(a, talk, (float*)out, H, KV, hd);
+    if (out_dtype == TP_BF16) talk_mix_k<bf16_t><<<dim3(M, H), 128, 0, s>>>(a, talk, (bf16_t*)out, H, KV, hd);
+    else if (out_dtype == TP_F32) talk_mix_k<float><<<dim3(M, H), 128, 0, s>>>(a, talk, (float*)out, H, KV, hd);
     else return tp_fail("talk_mix: unknown dtype %d", out_dtype);
     return tp_check_launch("talk_mix");
 }

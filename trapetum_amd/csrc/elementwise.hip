@@ -687,24 +687,32 @@ extern "C" int tp_gated_act(const float* y, void* out, int dtype, int M, int I, 
 // rows float32 or bf16 [M, N], out in its own dtype; act 0: none, 1: the exact gelu, x Phi(x) = 0.5 x (1 + erf(x / sqrt 2)).
 enum { TP_BIAS_NONE = 0, TP_BIAS_GELU_ERF = 1 };
 template <typename TI, typename TO>
-__global__ void bias_act_k(const TI* __restrict__ rows, const float* __restrict__ bias, TO* __restrict__ out, long total, int N, int act) {
+__global__ void bias_act_k(const TI* __restrict__ rows, const float* __restrict__ bias, TO* __restrict__ out, long total, int N, int pad, int act) {
+    const int W = N + pad;                               // the output's rows are wider by `pad`: a one, then zeros
     for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
-        float y = ld_f32(rows + i) + (bias ? bias[i % N] : 0.f);
-        if (act == TP_BIAS_GELU_ERF) y = 0.5f * y * (1.f + erff(y * 0.70710678118654752f));
+        const long r = i / W;
+        const int c = (int)(i - r * W);
+        float y = c == N ? 1.f : 0.f;
+        if (c < N) {
+            y = ld_f32(rows + r * N + c) + (bias ? bias[c] : 0.f);
+            if (act == TP_BIAS_GELU_ERF) y = 0.5f * y * (1.f + erff(y * 0.70710678118654752f));
+        }
         st_f32(out + i, y);
     }
 }
 
-extern "C" int tp_bias_act(const void* rows, int in_dtype, const float* bias, void* out, int out_dtype, int M, int N, int act, void* stream) {
-    TP_REQUIRE(rows && out && M > 0 && N > 0, "bias_act: empty shape M=%d N=%d", M, N);
+// pad > 0: the output has N + pad columns, column N holds ones and the rest zeros, so that the product that follows can
+// carry its bias as column N of its matrix
+extern "C" int tp_bias_act(const void* rows, int in_dtype, const float* bias, void* out, int out_dtype, int M, int N, int pad, int act, void* stream) {
+    TP_REQUIRE(rows && out && M > 0 && N > 0 && pad >= 0, "bias_act: empty shape M=%d N=%d pad=%d", M, N, pad);
     TP_REQUIRE(act == TP_BIAS_NONE || act == TP_BIAS_GELU_ERF, "bias_act: unknown activation %d", act);
-    const long total = (long)M * N;
+    const long total = (long)M * (N + pad);
     long blocks = (total + 255) / 256;
     if (blocks > 8192) blocks = 8192;
     hipStream_t s = (hipStream_t)stream;
-    if (in_dtype == TP_F32 && out_dtype == TP_F32) bias_act_k<float, float><<<(unsigned)blocks, 256, 0, s>>>((const float*)rows, bias, (float*)out, total, N, act);
-    else if (in_dtype == TP_F32 && out_dtype == TP_BF16) bias_act_k<float, bf16_t><<<(unsigned)blocks, 256, 0, s>>>((const float*)rows, bias, (bf16_t*)out, total, N, act);
-    else if (in_dtype == TP_BF16 && out_dtype == TP_BF16) bias_act_k<bf16_t, bf16_t><<<(unsigned)blocks, 256, 0, s>>>((const bf16_t*)rows, bias, (bf16_t*)out, total, N, act);
+    if (in_dtype == TP_F32 && out_dtype == TP_F32) bias_act_k<float, float><<<(unsigned)blocks, 256, 0, s>>>((const float*)rows, bias, (float*)out, total, N, pad, act);
+    else if (in_dtype == TP_F32 && out_dtype == TP_BF16) bias_act_k<float, bf16_t><<<(unsigned)blocks, 256, 0, s>>>((const float*)rows, bias, (bf16_t*)out, total, N, pad, act);
+    else if (in_dtype == TP_BF16 && out_dtype == TP_BF16) bias_act_k<bf16_t, bf16_t><<<(unsigned)blocks, 256, 0, s>>>((const bf16_t*)rows, bias, (bf16_t*)out, total, N, pad, act);
     else return tp_fail("bias_act: no kernel from dtype %d to dtype %d", in_dtype, out_dtype);
     return tp_check_launch("bias_act");
 }

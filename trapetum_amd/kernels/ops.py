@@ -36,7 +36,7 @@ _CORE_SIGS = {
     "tp_gated_act": [_P, _P, _I, _I, _I, _I, _F, _F, _P],
     "tp_linear": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _F, _F, _P, _L, _I, _I, _P],
     "tp_shift_mix": [_P, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P],
-    "tp_bias_act": [_P, _I, _P, _P, _I, _I, _I, _I, _P],
+    "tp_bias_act": [_P, _I, _P, _P, _I, _I, _I, _I, _I, _P],
     "tp_mul_sigmoid_heads": [_P, _L, _I, _P, _L, _I, _I, _I, _I, _P],
     "tp_qkv_prepare": [_P, _L, _I, _P, _I, _I, _I, _I, _I, _P, _I, _I, _F, _P, _P, _P, _P, _I, _P],
     "tp_pool_write": [_P, _L, _P, _L, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _I, _P, _P, _I, _P],
@@ -665,9 +665,10 @@ class HipOps:
                    x.shape[1] // heads, self._stream())
         return x
 
-    def bias_act(self, rows, bias, activation, out_dtype):
+    def bias_act(self, rows, bias, activation, out_dtype, pad=0):
         """act(rows + bias) in float32, rounded once to out_dtype: rows [M, N] float32 or bfloat16, bias float32 [N] or None;
-        activation: one of BIAS_ACTIVATIONS."""
+        activation: one of BIAS_ACTIVATIONS.  pad: the output has that many more columns, a one and then zeros (the product
+        that follows then carries its own bias as a column of its matrix)."""
         if activation not in BIAS_ACTIVATIONS:
             raise KernelError(f"bias_act: activation '{activation}' has no kernel ({', '.join(str(a) for a in BIAS_ACTIVATIONS)})")
         self._dev(rows, bias)
@@ -676,9 +677,9 @@ class HipOps:
         m, n = rows.shape
         if bias is not None and (bias.dtype != torch.float32 or bias.numel() != n or not bias.is_contiguous()):
             raise KernelError(f"bias_act: the bias must be contiguous float32 [{n}]")
-        out = torch.empty((m, n), dtype=out_dtype, device=self.device)
+        out = torch.empty((m, n + pad), dtype=out_dtype, device=self.device)
         self._call(self.lib, "tp_bias_act", rows.data_ptr(), _code(rows.dtype), bias.data_ptr() if bias is not None else None, out.data_ptr(),
-                   _code(out_dtype), m, n, BIAS_ACTIVATIONS[activation], self._stream())
+                   _code(out_dtype), m, n, int(pad), BIAS_ACTIVATIONS[activation], self._stream())
         return out
 
     MAX_SLICED_WIDTH = 8192        # widest row `add_rms_norm` takes in K slices
@@ -836,7 +837,8 @@ class HipOps:
                 raise KernelError("attention_pooled: the blocks' pools have the cache's page size, and blocks need a window")
         self_out = torch.empty((m, H, KV if all_values else 1, hd), dtype=torch.float32, device=self.device)
         pieces = all(t is None or (t.data_ptr() % 16 == 0) for t in (q, k, v)) and qs % 8 == 0 and ks % 8 == 0 and vs % 8 == 0
-        if max_count and not self.force_plain_attention and q.dtype == torch.bfloat16 and hd % 32 == 0 and hd <= 256 and pieces:
+        if max_count and not self.force_plain_attention and q.dtype == torch.bfloat16 and hd % 32 == 0 and hd <= 256 and pieces \
+                and page & (page - 1) == 0:
             self._call(self.attn_lib(hd), "tp_attn_pooled_tile", q.data_ptr(), qs, k.data_ptr(), ks, v.data_ptr(), vs, n, int(max_count), H, KV,
                        cu_rows.data_ptr(), new_len.data_ptr(), table.data_ptr(), table.shape[1], k_pool.data_ptr(), v_pool.data_ptr(), page,
                        rows_cap or 0, btable.data_ptr() if blocks else None, btable.shape[1] if blocks else 0,

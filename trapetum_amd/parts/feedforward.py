@@ -48,8 +48,12 @@ class GatedMLP(FeedForward):
 
 class BiasedMLP(FeedForward):
     """down(act(up x + b_up)) + b_down: one product up, one down, both with a bias, no gate.  The first product's
-    float32 sums take the bias and the activation before they are rounded; the second leaves float32 rows for the
-    residual add."""
+    float32 sums take the bias and the activation before they are rounded.  The second product carries its bias as a
+    further column of its matrix, met by a column of ones in the activations (where the bias is exact in the matrix's
+    width: a bfloat16 checkpoint's always is), so it is left to the block's add like any other product, in K slices where
+    it has them; otherwise the bias is added by a launch of its own."""
+
+    PAD = 64       # columns added to the second product's K: the bias and zeros (K stays a whole number of k steps)
 
     def __init__(self, hidden_size, intermediate_size, activation="gelu_erf", tensors=("up", "down"), bias_suffix=".b"):
         """activation: gelu_erf, the exact x Phi(x).  tensors: local names of the two matrices; a bias is named like its
@@ -67,12 +71,24 @@ class BiasedMLP(FeedForward):
     def bind(self, tensors, rt):
         self.rt = rt
         (up, dn), b = self.names, self.bias_suffix
-        self.w_up, self.w_down = rt.matrix(tensors[up]), rt.matrix(tensors[dn])
+        import torch
+        self.w_up = rt.matrix(tensors[up])
         self.b_up, self.b_down = tensors[up + b].float().contiguous(), tensors[dn + b].float().contiguous()
+        w_down, bias = tensors[dn], tensors[dn + b]
+        self.folded = bool(torch.equal(bias.to(w_down.dtype).float(), bias.float()))
+        if self.folded:
+            wide = torch.cat([w_down, bias.to(w_down.dtype).reshape(-1, 1), w_down.new_zeros((w_down.shape[0], self.PAD - 1))], dim=1)
+            self.w_down = rt.matrix(wide.contiguous())
+        else:
+            self.w_down = rt.matrix(w_down)
 
     def forward(self, ctx, x, out=None):
         import torch
-        act = ctx.ops.bias_act(ctx.ops.linear(x, self.w_up, torch.float32), self.b_up, self.activation, ctx.dtype)
+        up = ctx.ops.linear(x, self.w_up, torch.float32)
+        if self.folded:
+            act = ctx.ops.bias_act(up, self.b_up, self.activation, ctx.dtype, pad=self.PAD)
+            return ctx.ops.linear(act, self.w_down, ctx.dtype, defer=True)
+        act = ctx.ops.bias_act(up, self.b_up, self.activation, ctx.dtype)
         return ctx.ops.linear(act, self.w_down, torch.float32, bias=self.b_down)
 
 
