@@ -267,7 +267,7 @@ constexpr int KSTRIDE = HD + 8, ROWS_STAGE = CHUNK * (KSTRIDE + VSTRIDE) * 2;   
 constexpr int NLOAD = (CHUNK * PIECES + 255) / 256;                                // 16-byte pieces a thread moves per chunk and kind
 }
 
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256, 2)
 attn_pooled_rows_k(AttnPooledTileArgs a) {
     __shared__ __attribute__((aligned(16))) unsigned char lds[2 * ROWS_STAGE];
     const int seq = blockIdx.y, h = blockIdx.z / a.VG, c = blockIdx.z - h * a.VG;
@@ -407,21 +407,28 @@ _Pragma("unroll") \
                 ph.h[t * 4 + i] = hi;
                 pl.h[t * 4 + i] = f32_to_bf16(pr[t][i] - bf16_to_f32(hi));
             }
-        uint32_t vw[8][VT / 2];
+        // the value rows' elements in two halves of the output tiles, so that a wave keeps to 256 registers and two
+        // blocks share a CU
+        constexpr int HALVES = VT % 4 == 0 ? 2 : 1, VH = VT / HALVES;       // (a half holds whole pairs of tiles)
 #pragma unroll
-        for (int e = 0; e < 8; e++) {
-            const uint32_t* src = reinterpret_cast<const uint32_t*>(v_lds + ((e < 4 ? 0 : 12) + 4 * j + e) * VSTRIDE + col * VT);
+        for (int hf = 0; hf < HALVES; hf++) {
+            uint32_t vw[8][VH / 2];
 #pragma unroll
-            for (int x = 0; x < VT / 2; x++) vw[e][x] = src[x];
-        }
+            for (int e = 0; e < 8; e++) {
+                const uint32_t* src = reinterpret_cast<const uint32_t*>(v_lds + ((e < 4 ? 0 : 12) + 4 * j + e) * VSTRIDE + col * VT + hf * VH);
 #pragma unroll
-        for (int vt = 0; vt < VT; vt++) {
-            PtFrag vf;
+                for (int x = 0; x < VH / 2; x++) vw[e][x] = src[x];
+            }
 #pragma unroll
-            for (int e = 0; e < 8; e++) vf.h[e] = (bf16_t)(vw[e][vt >> 1] >> (16 * (vt & 1)));
-            acc[vt] *= alpha;
-            acc[vt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, ph.v, acc[vt], 0, 0, 0);
-            acc[vt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pl.v, acc[vt], 0, 0, 0);
+            for (int v2 = 0; v2 < VH; v2++) {
+                const int vt = hf * VH + v2;
+                PtFrag vf;
+#pragma unroll
+                for (int e = 0; e < 8; e++) vf.h[e] = (bf16_t)(vw[e][v2 >> 1] >> (16 * (v2 & 1)));
+                acc[vt] *= alpha;
+                acc[vt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, ph.v, acc[vt], 0, 0, 0);
+                acc[vt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pl.v, acc[vt], 0, 0, 0);
+            }
         }
     }
 #undef PT_LOAD
