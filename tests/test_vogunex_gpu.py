@@ -53,7 +53,7 @@ def pooled_attention(rt, H, G, dim, vdim, rot, size, pool, cap, scale=0.3, base=
 
 @pytest.mark.parametrize("H,G,dim,vdim,rot,size,pool,cap", [
     (4, 2, 16, 24, 8, 11, 3, 30.0), (3, 3, 24, 8, 24, 20, 5, 12.0), (2, 1, 32, 32, 16, 16, 16, None), (1, 1, 12, 12, 0, 1, 1, 5.0),
-    (6, 2, 64, 48, 32, 40, 8, 20.0), (8, 2, 128, 64, 64, 33, 4, 50.0), (2, 2, 40, 72, 40, 7, None, 9.0), (4, 1, 80, 96, 20, 64, 2, None),
+    (6, 2, 64, 80, 16, 40, 6, 18.0), (8, 2, 128, 64, 64, 33, 4, 50.0), (2, 2, 40, 72, 40, 7, None, 9.0), (4, 1, 80, 96, 20, 64, 2, None),
     (6, 3, 48, 130, 48, 1000, 7, 15.0), (3, 1, 16, 16, 4, 2, 30, 10.0)])
 def test_pooled_attention_part(rt, H, G, dim, vdim, rot, size, pool, cap):
     """Prompts, single tokens and portions down to two rows, two sequences side by side."""
@@ -198,7 +198,7 @@ def latent_part(rt, H, dim, rot_dim, vdim, rank, q_rank, dims, size, scale=0.3, 
 
 
 @pytest.mark.parametrize("H,dim,rot_dim,vdim,rank,q_rank,dims,size", [
-    (3, 16, 8, 12, 24, 20, 8, 13), (2, 8, 16, 16, 16, 12, 12, 18), (1, 10, 4, 10, 6, 6, 0, 1000), (6, 64, 16, 64, 128, 80, 16, 40),
+    (3, 16, 8, 12, 24, 20, 8, 13), (2, 8, 16, 16, 16, 12, 12, 18), (1, 10, 4, 10, 6, 6, 0, 1000), (6, 48, 16, 64, 112, 72, 16, 40),
     (5, 24, 2, 20, 14, 5, 2, 1), (4, 32, 16, 32, 48, 24, 8, 64), (16, 64, 32, 64, 96, 48, 32, 70), (2, 8, 8, 8, 8, 8, 8, 2)])
 def test_latent_attention_part(rt, H, dim, rot_dim, vdim, rank, q_rank, dims, size):
     part, W, sizes = latent_part(rt, H, dim, rot_dim, vdim, rank, q_rank, dims, size)
