@@ -192,9 +192,9 @@ _Pragma("unroll") \
         for (int t = 0; t < 2; t++)
 #pragma unroll
             for (int i = 0; i < 4; i++) {
-                const bf16_t hi = f32_to_bf16(pr[t][i]);
-                ph.h[t * 4 + i] = hi;
-                pl.h[t * 4 + i] = f32_to_bf16(pr[t][i] - bf16_to_f32(hi));
+                const __bf16 hi = (__bf16)pr[t][i];
+                ph.v[t * 4 + i] = hi;
+                pl.v[t * 4 + i] = (__bf16)(pr[t][i] - (float)hi);
             }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -209,15 +209,19 @@ _Pragma("unroll") \
 #pragma unroll
             for (int x = 0; x < VT / 2; x++) vw[e][x] = src[x];
         }
+        PtFrag vfs[VT];
 #pragma unroll
         for (int vt = 0; vt < VT; vt++) {
             PtFrag vf;
 #pragma unroll
             for (int e = 0; e < 8; e++) vf.h[e] = (bf16_t)(vw[e][vt >> 1] >> (16 * (vt & 1)));
+            vfs[vt] = vf;
             acc[vt] *= alpha;
             acc[vt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, ph.v, acc[vt], 0, 0, 0);
-            acc[vt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pl.v, acc[vt], 0, 0, 0);
         }
+#pragma unroll
+        for (int vt = 0; vt < VT; vt++)                   // the second terms afterwards: no instruction waits for the one before it
+            acc[vt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vfs[vt].v, pl.v, acc[vt], 0, 0, 0);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
     }
@@ -366,12 +370,15 @@ _Pragma("unroll") \
         for (int t = 0; t < 2; t++) {
             sc[t] = (pt_f32x4){0.f, 0.f, 0.f, 0.f};
             const bf16_t* krow = k_lds + (t * 16 + col) * KSTRIDE + j * 8;
+            pt_f32x4 odd = (pt_f32x4){0.f, 0.f, 0.f, 0.f};     // two chains of sums a tile: an instruction waits for every second one before it only
 #pragma unroll
             for (int s = 0; s < KS; s++) {
                 PtFrag kf;
                 kf.v = *reinterpret_cast<const pt_bf16x8*>(krow + s * 32);
-                sc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qf[s].v, sc[t], 0, 0, 0);
+                if (s & 1) odd = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qf[s].v, odd, 0, 0, 0);
+                else sc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qf[s].v, sc[t], 0, 0, 0);
             }
+            sc[t] += odd;
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 const int u = u0 + t * 16 + j * 4 + i, pos = LO + u - NB;
@@ -403,9 +410,9 @@ _Pragma("unroll") \
         for (int t = 0; t < 2; t++)
 #pragma unroll
             for (int i = 0; i < 4; i++) {
-                const bf16_t hi = f32_to_bf16(pr[t][i]);
-                ph.h[t * 4 + i] = hi;
-                pl.h[t * 4 + i] = f32_to_bf16(pr[t][i] - bf16_to_f32(hi));
+                const __bf16 hi = (__bf16)pr[t][i];
+                ph.v[t * 4 + i] = hi;
+                pl.v[t * 4 + i] = (__bf16)(pr[t][i] - (float)hi);
             }
         // the value rows' elements in two halves of the output tiles, so that a wave keeps to 256 registers and two
         // blocks share a CU
@@ -419,16 +426,20 @@ _Pragma("unroll") \
 #pragma unroll
                 for (int x = 0; x < VH / 2; x++) vw[e][x] = src[x];
             }
+            PtFrag vfs[VH];
 #pragma unroll
             for (int v2 = 0; v2 < VH; v2++) {
                 const int vt = hf * VH + v2;
                 PtFrag vf;
 #pragma unroll
                 for (int e = 0; e < 8; e++) vf.h[e] = (bf16_t)(vw[e][v2 >> 1] >> (16 * (v2 & 1)));
+                vfs[v2] = vf;
                 acc[vt] *= alpha;
                 acc[vt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, ph.v, acc[vt], 0, 0, 0);
-                acc[vt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pl.v, acc[vt], 0, 0, 0);
             }
+#pragma unroll
+            for (int v2 = 0; v2 < VH; v2++)               // the second terms afterwards: no instruction waits for the one before it
+                acc[hf * VH + v2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vfs[v2].v, pl.v, acc[hf * VH + v2], 0, 0, 0);
         }
     }
 #undef PT_LOAD
